@@ -158,3 +158,43 @@ class Attention(nn.Module):
                                    ctx.block_tables[:Bd], ctx.context_lens, self.scale,
                                    ctx.max_context_len, out=o[:Bd])
         return o.reshape(T, self.num_heads * self.head_dim)
+
+
+class SinkAttention(nn.Module):
+    """Causal attention over a paged cache whose softmax denominator carries one extra term
+    ``exp(sink_h)`` per query head (no key, no value), with key and value heads of different
+    sizes (K cache [blocks, block, G, D], V cache [blocks, block, G, E]) and an optional
+    per-head output gate ``sigmoid(gate_h)`` applied inside the kernel.  ``scale`` is the full
+    score multiplier.  Scores, weights and the weighted sum are fp32 in every implementation."""
+
+    def __init__(self, num_heads: int, num_kv_heads: int, head_dim: int, v_head_dim: int,
+                 scale: float):
+        super().__init__()
+        self.num_heads, self.num_kv_heads = num_heads, num_kv_heads
+        self.head_dim, self.v_head_dim, self.scale = head_dim, v_head_dim, scale
+        self.sink = nn.Parameter(torch.zeros(num_heads, dtype=torch.float32), requires_grad=False)
+        self.k_cache: Optional[torch.Tensor] = None
+        self.v_cache: Optional[torch.Tensor] = None
+
+    def forward(self, q: torch.Tensor, gate: Optional[torch.Tensor]) -> torch.Tensor:
+        """q [T,H,D] (rotated; rows may be strided), gate [T,H] raw or None; K/V of every token
+        of the step are in the cache already.  Returns [T, H*E]."""
+        ctx = get_context()
+        if self.k_cache is None:
+            raise RuntimeError("attention needs an allocated KV cache")
+        T = q.shape[0]
+        out = torch.zeros((T, self.num_heads, self.v_head_dim), dtype=q.dtype, device=q.device)
+        a = (self.k_cache, self.v_cache)
+        if not ctx.is_prefill:
+            ops.sink_attention_decode(q, *a, ctx.block_tables, ctx.context_lens, self.scale,
+                                      self.sink, gate, out)
+        else:
+            Bd = ctx.num_decode_seqs
+            if ctx.num_seqs > Bd:
+                ops.sink_attention_prefill(q, *a, ctx.cu_seqlens_q[Bd:], ctx.cu_seqlens_k[Bd:],
+                                           ctx.block_tables[Bd:], self.scale, self.sink, gate, out)
+            if Bd:
+                ops.sink_attention_decode(q[:Bd], *a, ctx.block_tables[:Bd], ctx.context_lens,
+                                          self.scale, self.sink,
+                                          None if gate is None else gate[:Bd], out[:Bd])
+        return out.view(T, self.num_heads * self.v_head_dim)

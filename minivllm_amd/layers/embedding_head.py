@@ -61,6 +61,8 @@ class VocabParallelEmbedding(nn.Module):
 class ParallelLMHead(VocabParallelEmbedding):
     def select_last(self, hidden: torch.Tensor) -> torch.Tensor:
         ctx = get_context()
+        if ctx.logit_rows is not None:
+            return hidden.index_select(0, ctx.logit_rows.long())
         if ctx.is_prefill and ctx.cu_seqlens_q is not None:
             last = (ctx.cu_seqlens_q[1:] - 1).long()
             hidden = hidden.index_select(0, last)
@@ -77,3 +79,24 @@ class ParallelLMHead(VocabParallelEmbedding):
             if logits is None:
                 return None
         return logits[..., :self.num_embeddings]
+
+
+class HashedBigramEmbedding(nn.Module):
+    """A second embedding table addressed by a hash of (previous token, token): row
+    ``(prev * mul_prev + token * mul_cur) mod buckets``; a sequence's first token uses the extra
+    row ``buckets``.  The rows are computed on the host while the batch is assembled
+    (``rows_for``: the previous token comes from the sequence's own token list, so a prompt cut
+    into portions needs no device-side state), the lookup is fused with the token embedding
+    (``ops.embed_sum``)."""
+
+    def __init__(self, buckets: int, embedding_dim: int, mul_prev: int, mul_cur: int):
+        super().__init__()
+        self.buckets, self.mul_prev, self.mul_cur = buckets, mul_prev, mul_cur
+        self.weight = nn.Parameter(torch.zeros(buckets + 1, embedding_dim), requires_grad=False)
+
+    def rows_for(self, tokens, prev_tokens):
+        """numpy int arrays: this step's tokens and the token before each (-1: none)."""
+        import numpy as np
+        t, p = np.asarray(tokens, np.int64), np.asarray(prev_tokens, np.int64)
+        rows = (p * self.mul_prev + t * self.mul_cur) % self.buckets
+        return np.where(p < 0, self.buckets, rows).astype(np.int32)

@@ -46,3 +46,18 @@ class RMSNorm(nn.Module):
 
 
 LayerNorm = RMSNorm      # the reference's class name
+
+
+class OffsetRMSNorm(nn.Module):
+    """RMS norm whose stored weight is an offset from one: ``x / rms(x) * (1 + weight)``.  The
+    weight stays fp32 whatever the activation dtype is; the op that applies it is chosen by the
+    caller (``ops.offset_rms_norm`` alone, or ``ops.post_norm_residual`` when the result is added
+    to a fp32 residual stream and the next sublayer's norm follows at once)."""
+
+    def __init__(self, hidden_size: int, eps: float = 1e-6):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.zeros(hidden_size, dtype=torch.float32), requires_grad=False)
+
+    def forward(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        return ops.offset_rms_norm(x, self.weight, self.eps, out_dtype or x.dtype)

@@ -44,3 +44,22 @@ class RotaryEmbedding(nn.Module):
 @lru_cache(maxsize=4)
 def get_rope(head_size: int, rotary_dim: int, max_position: int, base: float) -> RotaryEmbedding:
     return RotaryEmbedding(head_size, rotary_dim, max_position, base)
+
+
+class PairRotaryEmbedding(nn.Module):
+    """Rotation of neighbouring pairs (2i, 2i+1) of the first ``rotary_dim`` entries of a head
+    (the interleaved convention), the rest passing unchanged.  ``scaling``: None or a dict with
+    ``factor / low / high / original`` (the Llama 3.1 rule: wavelengths below original/high
+    keep their frequency, above original/low divide it by factor, a linear blend between).
+    Owns the fp32 table [max_position, rotary_dim] (cos, then sin) whose angles are formed in
+    fp32; the rotation itself happens in ``ops.pair_rope_mix_store``."""
+
+    def __init__(self, rotary_dim: int, max_position: int, base: float, scaling=None):
+        super().__init__()
+        if rotary_dim % 2:
+            raise ValueError("rotary_dim must be even")
+        self.rotary_dim = rotary_dim
+        from minivllm_amd.ops import torch_seqmix
+        self.register_buffer("cos_sin_cache",
+                             torch_seqmix.pair_cos_sin_table(rotary_dim, max_position, base, scaling),
+                             persistent=False)

@@ -226,3 +226,74 @@ def sample(logits, temperatures, seed=0, step=0, generator=None):
     if _on_gpu(logits):
         return _hip().sample(logits, temperatures, seed, step)
     return torch_ref.sample(logits, temperatures, generator)
+
+
+# ------------------------------------------------------------------ hybrid decoders
+# (fp32 residual stream with zero-centred norms, pair rotation + value mixing, attention with a
+# sink, gated delta rule, grouped expert routing).  GPU tensors go to the kernels of
+# ``csrc/hybrid`` (their own library, ``ops.hip_hybrid``), CPU tensors to ``torch_seqmix``.
+from . import torch_seqmix
+
+
+def _hybrid():
+    from . import hip_hybrid     # raises with a build hint when the library is absent
+    return hip_hybrid
+
+
+def _seqmix(t):
+    return _hybrid() if _on_gpu(t) else torch_seqmix
+
+
+def embed_sum(ids, aux_rows, table, aux_table):
+    return _seqmix(table).embed_sum(ids, aux_rows, table, aux_table)
+
+
+def offset_rms_norm(x, w, eps, out_dtype):
+    return _seqmix(x).offset_rms_norm(x, w, eps, out_dtype)
+
+
+def post_norm_residual(y, wb, x, eps, w_next, out_dtype):
+    return _seqmix(x).post_norm_residual(y, wb, x, eps, w_next, out_dtype)
+
+
+def pair_rope_mix_store(q, k, v, positions, cos_sin, rot_dims, v_first, lam, v_mode,
+                        k_cache, v_cache, slot_mapping):
+    return _seqmix(q).pair_rope_mix_store(q, k, v, positions, cos_sin, rot_dims, v_first, lam,
+                                          v_mode, k_cache, v_cache, slot_mapping)
+
+
+def sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables, scale, sink, gate, out):
+    return _seqmix(q).sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables,
+                                             scale, sink, gate, out)
+
+
+def sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens, scale, sink, gate, out):
+    return _seqmix(q).sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens,
+                                            scale, sink, gate, out)
+
+
+def delta_prepare(q, k, v, b, a, wq, wk, wv, a_log, dt_bias, conv_state, cu_q, positions, slots,
+                  row_seq=None):
+    """``row_seq`` [T] (GPU, prefill-form steps): the sequence of each row, -1 for rows that
+    belong to none; the CPU form walks ``cu_q`` instead."""
+    if _on_gpu(q):
+        return _hybrid().delta_prepare(q, k, v, b, a, wq, wk, wv, a_log, dt_bias, conv_state,
+                                       cu_q, positions, slots, row_seq)
+    return torch_seqmix.delta_prepare(q, k, v, b, a, wq, wk, wv, a_log, dt_bias, conv_state,
+                                      cu_q, positions, slots)
+
+
+def delta_scan(qn, kn, vv, beta, decay, state, cu_q, positions, slots):
+    return _seqmix(qn).delta_scan(qn, kn, vv, beta, decay, state, cu_q, positions, slots)
+
+
+def gated_head_norm(o, w, gate, eps, out_dtype):
+    return _seqmix(o).gated_head_norm(o, w, gate, eps, out_dtype)
+
+
+def grouped_route(h, router_w, top, groups, keep):
+    return _seqmix(h).grouped_route(h, router_w, top, groups, keep)
+
+
+def gelu_route_scale(up, dense, ff, out_dtype):
+    return _seqmix(up).gelu_route_scale(up, dense, ff, out_dtype)

@@ -1,0 +1,246 @@
+"""Plain PyTorch forms of the ops that hybrid decoders add to the dense ones: norms with a
+zero-centred weight around a fp32 residual stream, rotation of neighbouring pairs with value
+mixing, attention with a sink term and separate key / value head sizes, the gated delta rule
+with its short convolutions, and routing over grouped experts.  They run CPU tensors (the
+engine's CPU mode) and serve as the shape-for-shape counterpart of the gfx950 kernels in
+``csrc/hybrid`` (``ops.hip_hybrid``).  Everything a recurrence touches is fp32 here too.
+
+Sequence layout arguments shared by the per-sequence ops (``SeqLayout``): ``cu_q`` [B+1] rows
+of each sequence inside the step (None: row b is sequence b, one token each), ``positions`` [T]
+(a sequence's first row holds the position where this step starts it), ``slots`` [B] state slot
+per sequence (negative: an unused row of a padded batch).
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+import torch.nn.functional as F
+
+from .torch_ref import _gather_paged
+
+
+def _bounds(cu_q, positions, B):
+    if cu_q is None:
+        rows = list(range(B + 1))
+    else:
+        rows = cu_q.tolist()
+    return rows
+
+
+# ------------------------------------------------------------------ embedding + norms
+def embed_sum(ids, aux_rows, table, aux_table):
+    """fp32 rows ``table[ids] + aux_table[aux_rows]`` (``aux_table`` None: the first alone)."""
+    x = table[ids.long()].float()
+    if aux_table is not None:
+        x = x + aux_table[aux_rows.long()].float()
+    return x
+
+
+def offset_rms_norm(x, w, eps, out_dtype):
+    xf = x.float()
+    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * (1.0 + w.float())).to(out_dtype)
+
+
+def post_norm_residual(y, wb, x, eps, w_next, out_dtype):
+    """``x += norm(y) * (1 + wb)`` in place on the fp32 stream ``x``; with ``w_next`` also returns
+    ``norm(x) * (1 + w_next)`` (the input of the next sublayer)."""
+    yf = y.float()
+    x.add_(yf * torch.rsqrt(yf.pow(2).mean(-1, keepdim=True) + eps) * (1.0 + wb.float()))
+    if w_next is None:
+        return None
+    return offset_rms_norm(x, w_next, eps, out_dtype)
+
+
+# ------------------------------------------------------------------ rotation, value mix, store
+def pair_cos_sin_table(rot_dims: int, max_position: int, base: float, scaling) -> torch.Tensor:
+    """[max_position, rot_dims] fp32: cos of the rot_dims/2 angles, then their sin.  The angle
+    position * f_i is formed in fp32 (f_i rounded to fp32 first), its cos / sin in fp64."""
+    import math
+    i = torch.arange(rot_dims // 2, dtype=torch.float64)
+    f = base ** (-2.0 * i / rot_dims)
+    if scaling:
+        factor, low, high = float(scaling["factor"]), float(scaling["low"]), float(scaling["high"])
+        orig = float(scaling["original"])
+        wl = 2 * math.pi / f
+        s = (orig / wl - low) / (high - low)
+        mid = (1 - s) * f / factor + s * f
+        f = torch.where(wl < orig / high, f, torch.where(wl > orig / low, f / factor, mid))
+    ang = torch.arange(max_position, dtype=torch.float32)[:, None] * f.float()[None, :]
+    ang = ang.double()
+    return torch.cat([ang.cos(), ang.sin()], -1).float()
+
+
+def _rotate_pairs(x, cs, rot_dims):
+    """x [T, heads, D] fp32, cs [T, rot_dims] -> rotated copy."""
+    if rot_dims == 0:
+        return x
+    half = rot_dims // 2
+    c, s = cs[:, None, :half], cs[:, None, half:]
+    a, b = x[..., 0:rot_dims:2], x[..., 1:rot_dims:2]
+    out = x.clone()
+    out[..., 0:rot_dims:2] = a * c - b * s
+    out[..., 1:rot_dims:2] = b * c + a * s
+    return out
+
+
+def pair_rope_mix_store(q, k, v, positions, cos_sin, rot_dims, v_first, lam, v_mode,
+                        k_cache, v_cache, slot_mapping):
+    """q [T,H,D], k [T,G,D], v [T,G,E] views of a projection output.  Rotates q in place and k
+    on its way into the cache; ``v_mode`` 1: copies v into ``v_first``; 2: v <- (1 - lam) v +
+    lam v_first (fp32); the result goes into the cache.  Rows with slot < 0 store nothing."""
+    cs = cos_sin[positions.long()] if rot_dims else None
+    q.copy_(_rotate_pairs(q.float(), cs, rot_dims).to(q.dtype))
+    kr = _rotate_pairs(k.float(), cs, rot_dims)
+    vf = v.float()
+    if v_mode == 1:
+        v_first.copy_(v.reshape(v_first.shape))
+    elif v_mode == 2:
+        lf = lam.float()
+        vf = (1.0 - lf) * vf + lf * v_first.float().reshape(vf.shape)
+    if k_cache is not None and slot_mapping is not None:
+        bs = k_cache.shape[1]
+        slots = slot_mapping.long()
+        keep = slots >= 0
+        blk, off = torch.div(slots[keep], bs, rounding_mode="floor"), slots[keep] % bs
+        k_cache[blk, off] = kr[keep].to(k_cache.dtype)
+        v_cache[blk, off] = vf[keep].to(v_cache.dtype)
+
+
+# ------------------------------------------------------------------ attention with a sink
+def _sink_attend(q, k, v, scale, sink, gate, offset):
+    """q [Lq,H,D], k [Lk,G,D], v [Lk,G,E], gate [Lq,H] -> [Lq,H,E] fp32."""
+    Lq, H, _ = q.shape
+    Lk, G, _ = k.shape
+    r = H // G
+    qf = q.float().transpose(0, 1)
+    kf = k.float().transpose(0, 1).repeat_interleave(r, 0)
+    vf = v.float().transpose(0, 1).repeat_interleave(r, 0)
+    s = torch.matmul(qf, kf.transpose(1, 2)) * scale                  # [H, Lq, Lk]
+    qi = torch.arange(Lq)[:, None] + offset
+    s = s.masked_fill((torch.arange(Lk)[None, :] > qi)[None], float("-inf"))
+    s = torch.cat([s, sink.float()[:, None, None].expand(H, Lq, 1)], -1)
+    p = torch.softmax(s, -1)[..., :Lk]
+    o = torch.matmul(p, vf).transpose(0, 1)                           # [Lq, H, E]
+    if gate is not None:
+        o = o * torch.sigmoid(gate.float())[:, :, None]
+    return o
+
+
+def sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables, scale, sink, gate, out):
+    cq, ck = cu_q.tolist(), cu_k.tolist()
+    for b in range(len(cq) - 1):
+        s, e = cq[b], cq[b + 1]
+        lk = ck[b + 1] - ck[b]
+        if e == s:
+            continue
+        k = _gather_paged(k_cache, block_tables[b], lk)
+        v = _gather_paged(v_cache, block_tables[b], lk)
+        out[s:e] = _sink_attend(q[s:e], k, v, scale, sink, None if gate is None else gate[s:e],
+                                lk - (e - s)).to(out.dtype)
+    return out
+
+
+def sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens, scale, sink, gate, out):
+    for b, L in enumerate(context_lens.tolist()):
+        if L <= 0:
+            continue
+        k = _gather_paged(k_cache, block_tables[b], L)
+        v = _gather_paged(v_cache, block_tables[b], L)
+        out[b:b + 1] = _sink_attend(q[b:b + 1], k, v, scale, sink,
+                                    None if gate is None else gate[b:b + 1], L - 1).to(out.dtype)
+    return out
+
+
+# ------------------------------------------------------------------ gated delta rule
+def delta_prepare(q, k, v, b, a, wq, wk, wv, a_log, dt_bias, conv_state, cu_q, positions, slots):
+    """Short causal convolution + silu on q / k / v (their last taps-1 inputs per sequence live
+    in ``conv_state`` [slots, taps-1, Cq+Ck+Cv] fp32 and are replaced by this step's), unit
+    vectors for q (times D^-1/2) and k, beta = sigmoid(b), decay = exp(-exp(A_log) softplus(a +
+    dt_bias)).  q, k [T,G,D]; v [T,H,E]; b, a [T,H].  Returns fp32 (q, k, v, beta, decay)."""
+    T, G, D = q.shape
+    H, E = v.shape[1], v.shape[2]
+    x = torch.cat([q.reshape(T, -1), k.reshape(T, -1), v.reshape(T, -1)], -1).float()
+    w = torch.cat([wq, wk, wv], 0).float()                             # [C, taps]
+    taps = w.shape[1]
+    y = torch.empty_like(x)
+    B = slots.shape[0]
+    rows = _bounds(cu_q, positions, B)
+    for i in range(B):
+        s, e, slot = rows[i], rows[i + 1], int(slots[i])
+        if e == s or slot < 0:
+            continue
+        if taps > 1:
+            tail = conv_state[slot] if int(positions[s]) > 0 else torch.zeros_like(conv_state[slot])
+            full = torch.cat([tail, x[s:e]], 0)
+            conv_state[slot] = full[full.shape[0] - (taps - 1):]
+        else:
+            full = x[s:e]
+        win = full.unfold(0, taps, 1)                                  # [n, C, taps]
+        y[s:e] = (win * w[None]).sum(-1)
+    y = F.silu(y)
+    cq, ckk = G * D, 2 * G * D
+    qn, kn, vv = y[:, :cq].view(T, G, D), y[:, cq:ckk].view(T, G, D), y[:, ckk:].view(T, H, E)
+    qn = qn * torch.rsqrt(qn.pow(2).sum(-1, keepdim=True) + 1e-6) * D ** -0.5
+    kn = kn * torch.rsqrt(kn.pow(2).sum(-1, keepdim=True) + 1e-6)
+    beta = torch.sigmoid(b.float())
+    decay = torch.exp(-torch.exp(a_log.float()) * F.softplus(a.float() + dt_bias.float()))
+    return qn, kn, vv.contiguous(), beta, decay
+
+
+def delta_scan(qn, kn, vv, beta, decay, state, cu_q, positions, slots):
+    """Per sequence and head, token after token: S <- decay S; u = beta (v - S^T k); S <- S + k
+    u^T; o = S^T q.  ``state`` [slots, H, D, E] fp32 is read (zeros where the sequence starts at
+    position 0) and left holding the state after the step.  Returns o [T,H,E] fp32."""
+    T, G, D = qn.shape
+    H, E = vv.shape[1], vv.shape[2]
+    r = H // G
+    o = torch.zeros(T, H, E, dtype=torch.float32)
+    B = slots.shape[0]
+    rows = _bounds(cu_q, positions, B)
+    qh, kh = qn.repeat_interleave(r, 1), kn.repeat_interleave(r, 1)
+    for i in range(B):
+        s, e, slot = rows[i], rows[i + 1], int(slots[i])
+        if e == s or slot < 0:
+            continue
+        S = state[slot].clone() if int(positions[s]) > 0 else torch.zeros(H, D, E)
+        for t in range(s, e):
+            S = S * decay[t][:, None, None]
+            u = beta[t][:, None] * (vv[t] - torch.einsum("hde,hd->he", S, kh[t]))
+            S = S + kh[t][:, :, None] * u[:, None, :]
+            o[t] = torch.einsum("hde,hd->he", S, qh[t])
+        state[slot] = S
+    return o
+
+
+def gated_head_norm(o, w, gate, eps, out_dtype):
+    """o [T,H,E] fp32 / rms over E * w[E] * silu(gate [T,H,E])."""
+    y = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+    return (y * F.silu(gate.float()).view(o.shape)).to(out_dtype)
+
+
+# ------------------------------------------------------------------ grouped expert routing
+def grouped_route(h, router_w, top, groups, keep):
+    """Softmax over all experts in fp32; only experts of the ``keep`` groups (of ``groups``
+    equal runs of neighbours) whose best score is largest are eligible; the ``top`` largest
+    eligible scores, unnormalised, are the weights.  Returns [T, experts] fp32, zero elsewhere."""
+    z = h.float() @ router_w.float().t()
+    s = torch.softmax(z, -1)
+    T, E = s.shape
+    per = E // groups
+    best = s.view(T, groups, per).max(-1).values
+    # ties go to the lower index, as in the kernel: rank by (score desc, index asc)
+    kept = torch.zeros(T, groups, dtype=torch.bool)
+    kept.scatter_(1, torch.sort(best, dim=-1, descending=True, stable=True).indices[:, :keep], True)
+    masked = torch.where(kept.repeat_interleave(per, 1), s, torch.full_like(s, -1.0))
+    ids = torch.sort(masked, dim=-1, descending=True, stable=True).indices[:, :top]
+    dense = torch.zeros_like(s)
+    dense.scatter_(1, ids, s.gather(1, ids))
+    return dense
+
+
+def gelu_route_scale(up, dense, ff, out_dtype):
+    """up [T, experts*ff] -> gelu(up) * dense[t, expert] (exact erf gelu, fp32 math)."""
+    T = up.shape[0]
+    y = F.gelu(up.float()).view(T, -1, ff) * dense[:, :, None]
+    return y.view(T, -1).to(out_dtype)

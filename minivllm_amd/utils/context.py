@@ -40,6 +40,15 @@ class Context:
     # prefill: every query's position is its place in its context (k_len - q_len + i); the GPU
     # attention kernel then derives the rotary positions instead of loading them
     positions_in_context: bool = False
+    # models with per-sequence recurrent state: the state slot of each sequence of the step
+    # [B] (-1: an unused row of a padded batch), the sequence of each row [T] (-1: none; prefill
+    # form only), and per-token rows of an auxiliary embedding table the host worked out
+    state_slots: Optional[torch.Tensor] = None
+    row_seq: Optional[torch.Tensor] = None
+    aux_rows: Optional[torch.Tensor] = None
+    # rows whose logits the step wants instead of each sequence's last one (scoring a given
+    # text: every asked position of a prompt portion)
+    logit_rows: Optional[torch.Tensor] = None
 
 
 _CONTEXT = Context()

@@ -76,16 +76,25 @@ class _Stream:
 
 
 def load_weights_from_checkpoint(model: nn.Module, path: str) -> int:
-    """Load a HF Qwen3 checkpoint directory (safetensors) into ``model``."""
+    """Load a checkpoint directory (safetensors) into ``model``: through the model's own
+    ``load_weights`` when it has one (families whose tensor names are packed into fused
+    parameters their own way), else by the HF names and the packed-module mapping."""
+    if hasattr(model, "load_weights"):
+        return model.load_weights(iter_safetensors(path))
     return load_state_dict_into(model, _Stream(iter_safetensors(path)))
 
 
 def model_config_from_hf(path: str):
     """Build a ModelConfig from a HF ``config.json`` (model_type qwen3, qwen2, llama, mistral:
     the same decoder with or without QKV bias / per-head q,k norm)."""
-    from minivllm_amd.config import ModelConfig
     with open(os.path.join(path, "config.json")) as f:
         c = json.load(f)
+    return model_config_from_dict(c, os.path.basename(os.path.normpath(path)))
+
+
+def model_config_from_dict(c: dict, name: str = "model"):
+    """``model_config_from_hf`` for an already parsed ``config.json``."""
+    from minivllm_amd.config import ModelConfig
     heads = c["num_attention_heads"]
     kind = c.get("model_type", "qwen3")
     if kind not in ("qwen3", "qwen2", "llama", "mistral"):
@@ -111,4 +120,4 @@ def model_config_from_hf(path: str):
         qkv_bias=c.get("attention_bias", kind == "qwen2"), ffn_bias=c.get("mlp_bias", False),
         base=theta, max_position=c.get("max_position_embeddings", 40960),
         tie_word_embeddings=c.get("tie_word_embeddings", False),
-        name=os.path.basename(os.path.normpath(path)))
+        name=name)
