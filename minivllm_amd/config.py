@@ -277,17 +277,20 @@ class EngineConfig:
             raise ValueError("tp_shard_rank must be in [0, tp_shard)")
         if self.block_size <= 0 or (self.block_size & (self.block_size - 1)):
             raise ValueError(f"block_size must be a power of two, got {self.block_size}")
-        if m.num_heads % m.num_kv_heads:
-            raise ValueError("num_heads must be a multiple of num_kv_heads")
-        tp = self.tp_degree
-        if m.num_heads % tp or m.num_kv_heads % tp:
-            raise ValueError(
-                f"tensor-parallel degree {tp} must divide num_heads={m.num_heads} and "
-                f"num_kv_heads={m.num_kv_heads} (KV-head replication is not supported)")
-        if m.intermediate_size % tp:
-            raise ValueError("the tensor-parallel degree must divide intermediate_size")
-        if m.head_dim not in (64, 128) and self.resolved_device() == "cuda":
-            raise ValueError("HIP attention kernels support head_dim 64 and 128")
+        if hasattr(m, "validate_engine"):
+            m.validate_engine(self)      # a family with its own layer make-up checks itself
+        else:
+            if m.num_heads % m.num_kv_heads:
+                raise ValueError("num_heads must be a multiple of num_kv_heads")
+            tp = self.tp_degree
+            if m.num_heads % tp or m.num_kv_heads % tp:
+                raise ValueError(
+                    f"tensor-parallel degree {tp} must divide num_heads={m.num_heads} and "
+                    f"num_kv_heads={m.num_kv_heads} (KV-head replication is not supported)")
+            if m.intermediate_size % tp:
+                raise ValueError("the tensor-parallel degree must divide intermediate_size")
+            if m.head_dim not in (64, 128) and self.resolved_device() == "cuda":
+                raise ValueError("HIP attention kernels support head_dim 64 and 128")
         if self.max_model_length > m.max_position:
             raise ValueError(
                 f"max_model_length={self.max_model_length} exceeds the RoPE table "
@@ -317,7 +320,8 @@ class EngineConfig:
         Unknown keys raise, so typos do not silently fall back to defaults.
         """
         cfg = dict(cfg)
-        if isinstance(cfg.get("model"), ModelConfig):
+        if cfg.get("model") is not None and not isinstance(cfg["model"], dict):
+            # a configuration object: ModelConfig, or another family's (models/registry.py)
             model = cfg.pop("model")
         else:
             preset = cfg.pop("model_preset", None)

@@ -40,7 +40,10 @@ class Block:
 
 
 class BlockManager:
-    def __init__(self, num_blocks: int, block_size: int):
+    def __init__(self, num_blocks: int, block_size: int, prefix_caching: bool = True):
+        # off: no block is ever found through its hash or published under one (models whose
+        # layers also carry recurrent state cannot resume from cached KV blocks alone)
+        self.prefix_caching = prefix_caching
         if num_blocks <= 0:
             raise ValueError("num_blocks must be positive")
         self.block_size = block_size
@@ -108,7 +111,7 @@ class BlockManager:
         seq.num_cached_tokens = 0
         for i in range(seq.num_blocks):
             token_ids = seq.block(i)
-            full = len(token_ids) == bs
+            full = len(token_ids) == bs and self.prefix_caching
             h = self.compute_hash(token_ids, h) if full else -1
             block_id = self.hash_to_block_id.get(h, -1) if full else -1
             if full:
@@ -173,7 +176,7 @@ class BlockManager:
             block = self._fresh_block()
             seq.block_table.append(block.block_id)
         assert len(seq.block_table) == seq.num_blocks
-        if seq.num_tokens % bs == 0:
+        if seq.num_tokens % bs == 0 and self.prefix_caching:
             # this step fills the last block: publish it for prefix sharing
             last = self.blocks[seq.block_table[-1]]
             if last.hash == -1:
@@ -183,6 +186,15 @@ class BlockManager:
                     h = self.compute_hash(token_ids, prefix)
                     last.update(h, token_ids)
                     self.hash_to_block_id[h] = last.block_id
+
+    def can_grow(self, seq: Sequence) -> bool:
+        return len(self.free_block_ids) >= seq.num_blocks - len(seq.block_table)
+
+    def grow(self, seq: Sequence) -> None:
+        """Fresh blocks for every token the sequence has gained since its table was last
+        brought up to date (a text fed in portions); nothing is published."""
+        while len(seq.block_table) < seq.num_blocks:
+            seq.block_table.append(self._fresh_block().block_id)
 
     def append_ahead(self, seq: Sequence) -> None:
         """Give ``seq`` the block that the token AFTER its newest one starts, if it has none yet
@@ -365,10 +377,13 @@ class NativeBlockManager:
                 "prefix_hit_rate": hits / queries if queries else 0.0}
 
 
-def make_block_manager(num_blocks: int, block_size: int, native: Optional[bool] = None):
+def make_block_manager(num_blocks: int, block_size: int, native: Optional[bool] = None,
+                       prefix_caching: bool = True):
     """The C++ allocator when its library is built (default), else the Python one.
     ``MINIVLLM_PY_HOST=1`` forces the Python implementation."""
     import os
     if native is None:
         native = os.environ.get("MINIVLLM_PY_HOST") != "1" and _host_lib() is not None
+    if not prefix_caching:       # the Python allocator is the one that can run without hashes
+        return BlockManager(num_blocks, block_size, prefix_caching=False)
     return NativeBlockManager(num_blocks, block_size) if native else BlockManager(num_blocks, block_size)

@@ -95,7 +95,10 @@ class LLMEngine:
                                    max_prefill_delay_s=cfg.max_prefill_delay_ms / 1e3,
                                    enable_mixed_batches=cfg.enable_mixed_batches,
                                    ahead_over_block_edges=(cfg.decode_prelaunch_edges and os.environ.get(
-                                       "MINIVLLM_NO_EDGE_PRELAUNCH") != "1"))
+                                       "MINIVLLM_NO_EDGE_PRELAUNCH") != "1"),
+                                   num_state_slots=self.model_runner.num_state_slots,
+                                   prefix_caching=not self.model_runner.num_state_slots)
+        self._given: Dict[str, Sequence] = {}
         self.tokenizer = load_tokenizer(cfg.model_name_or_path, cfg.model.vocab_size)
         self.stats = EngineStats()
         self._exited = False
@@ -245,6 +248,49 @@ class LLMEngine:
         finished = self.scheduler.postprocess(seqs, token_ids)
         self._drop_stale_prelaunch()
         return ([(s.seq_id, s.completion_token_ids) for s in finished], num_tokens, is_prefill)
+
+    # ------------------------------------------------------ scoring given text
+    def score_step(self, entries, end=()) -> Dict[str, "torch.Tensor"]:
+        """One step of a given schedule over given tokens.  ``entries``: dicts with ``id`` (any
+        hashable name of a request), ``tokens`` (its next tokens; the request is admitted at its
+        first entry) and ``want`` (offsets among these tokens whose logits are asked for);
+        ``end``: names of the requests that are finished after this step (their KV blocks and
+        state slot go back to the pools).  All entries run as one batch through the scheduler's
+        admission (``Scheduler.schedule_given``) and the runner's ordinary step
+        (``ModelRunner.score``): portions of prompts as prefill rows, single next tokens of
+        running requests as decode rows.  Returns id -> fp32 logits [asked, vocab]."""
+        vocab = self.cfg.model.vocab_size
+        portions, want, names = [], {}, {}
+        for e in entries:
+            toks = [int(t) for t in e["tokens"]]
+            if not toks or any(t < 0 or t >= vocab for t in toks):
+                raise ValueError("an entry needs tokens inside the model vocabulary")
+            seq = self._given.get(e["id"])
+            if seq is None:
+                seq = Sequence(toks, SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True),
+                               block_size=self.cfg.block_size)
+                seq.block_size = self.cfg.block_size
+                self.scheduler.waiting.append(seq)
+                self._given[e["id"]] = seq
+            else:
+                seq.extend_tokens(toks)
+            if seq.num_tokens > self.cfg.max_model_length:
+                raise ValueError("the request outgrows max_model_length")
+            portions.append((seq, len(toks)))
+            want[seq.seq_id] = list(e.get("want", ()))
+            names[seq.seq_id] = e["id"]
+        out = {}
+        if portions:
+            self._check_workers()
+            seqs, is_prefill, riders = self.scheduler.schedule_given(portions)
+            got = self.model_runner.score(seqs, is_prefill, riders, want)
+            self.scheduler.advance_given(seqs)
+            out = {names[sid]: lg for sid, lg in got.items()}
+        for name in end:
+            seq = self._given.pop(name, None)
+            if seq is not None:
+                self.scheduler.release(seq)
+        return out
 
     def _drop_stale_prelaunch(self) -> None:
         """A decode step launched ahead whose sequences have all just finished would otherwise

@@ -35,7 +35,7 @@ from minivllm_amd.config import EngineConfig, as_engine_config
 from minivllm_amd.engine.rpc import ShmBroadcastChannel
 from minivllm_amd.engine.sequence import Sequence
 from minivllm_amd.layers.sampler import SamplerLayer
-from minivllm_amd.models.qwen3 import Qwen3ForCausalLM
+from minivllm_amd.models.registry import model_class_for
 from minivllm_amd.parallel import group as pg
 from minivllm_amd.utils.context import reset_context, set_context
 from minivllm_amd.utils.profiling import trace_range
@@ -165,7 +165,7 @@ class ModelRunner:
         torch.set_default_dtype(self.dtype)
         try:
             with torch.device(self.device):
-                self.model = Qwen3ForCausalLM(cfg.model)
+                self.model = model_class_for(cfg.model)(cfg.model)
         finally:
             torch.set_default_dtype(prev)
         self.model.eval()
@@ -174,10 +174,15 @@ class ModelRunner:
             load_weights_from_checkpoint(self.model, cfg.checkpoint_path)
         else:
             self.model.init_random_weights(cfg.seed)
+        # models that bring their own cache layout (attention layers with their own head sizes,
+        # layers with per-sequence recurrent state): see ``allocate_kv_cache``
+        self.hybrid = hasattr(self.model, "state_layers")
+        self.needs_aux_rows = hasattr(self.model, "aux_embedding_rows")
+        self.num_state_slots = cfg.max_num_sequences if self.hybrid and self.model.state_layers() else 0
         fold = cfg.fold_norm_weights
         if fold is None:
             fold = self.tp == 1 and not pg.collectives_active()
-        self.norms_folded = bool(self.on_gpu and fold)
+        self.norms_folded = bool(self.on_gpu and fold and not self.hybrid)
         if self.norms_folded:
             self.model.fold_norm_weights()
         self.sampler = SamplerLayer(seed=cfg.seed)
@@ -197,7 +202,7 @@ class ModelRunner:
 
         with torch.inference_mode():
             self.warmup_model()
-            if self.on_gpu and (cfg.tune_decode_gemms or cfg.tune_prefill_gemms):
+            if self.on_gpu and (cfg.tune_decode_gemms or cfg.tune_prefill_gemms) and not self.hybrid:
                 self._choose_gemm_kernels()
             self.allocate_kv_cache()
             if self.on_gpu and not self.enforce_eager:
@@ -353,7 +358,7 @@ class ModelRunner:
     def _init_buffers(self) -> None:
         cfg = self.cfg
         mb, MB = self.max_bs, self.max_blocks_per_seq
-        if self.on_gpu:
+        if self.on_gpu and not self.hybrid:
             # scratch the decode kernel needs to exist before any graph is captured
             from minivllm_amd.ops import hip
             groups = -(-(cfg.model.num_heads // cfg.model.num_kv_heads) // 16)
@@ -364,7 +369,7 @@ class ModelRunner:
         off = 0
         for name, n in (("input_ids", mb), ("positions", mb), ("slot_mapping", mb),
                         ("context_lens", mb), ("temperatures", mb), ("misc", 4),
-                        ("block_tables", mb * MB)):
+                        ("aux_rows", mb), ("state_slots", mb), ("block_tables", mb * MB)):
             self._dec_off[name] = (off, n)
             off += (n + 3) // 4 * 4
         self._dec_words = off
@@ -402,8 +407,8 @@ class ModelRunner:
         self._last_step_logits: Optional[torch.Tensor] = None
         self.prefill_graph_replays = 0
         pg_max, self.pg_max_seqs = cfg.prefill_graph_limits()
-        if not self.on_gpu or cfg.enforce_eager:
-            pg_max = 0
+        if not self.on_gpu or cfg.enforce_eager or self.hybrid:
+            pg_max = 0           # (hybrid models: prefill and mixed steps launch eagerly)
         pg_max = int(os.environ.get("MINIVLLM_PREFILL_GRAPH_MAX", pg_max))
         pg_max = min(pg_max, 4096, cfg.max_num_batched_tokens)
         self.pg_max_seqs = min(self.pg_max_seqs, cfg.max_num_sequences)
@@ -508,8 +513,11 @@ class ModelRunner:
         self._pg_logits, self._graph_logits, self._last_logits = {}, {}, None
         self._last_step_logits = None
         self.graph_pool = None
-        for layer in self.model.model.layers:
-            layer.self_attn.attn.k_cache = layer.self_attn.attn.v_cache = None
+        for attn in self._attention_modules():
+            attn.k_cache = attn.v_cache = None
+        if self.hybrid:
+            for d in self.model.state_layers():
+                d.state = d.conv_state = None
         self.kv_cache = None
         self.model = None
         self._dec_dev = self._pre_dev = None
@@ -550,8 +558,8 @@ class ModelRunner:
         """One prefill of the largest batch the scheduler can emit, without a KV cache, so
         that peak activation memory is known before the cache is sized
         (reference: model_runner.py:129-137)."""
-        if not self.on_gpu:
-            return
+        if not self.on_gpu or self.hybrid:
+            return               # (hybrid models size their caches from a fixed head-room)
         cfg = self.cfg
         torch.cuda.empty_cache()
         torch.cuda.reset_peak_memory_stats()
@@ -572,9 +580,20 @@ class ModelRunner:
         torch.cuda.synchronize()
 
     # ================================================================ KV cache
+    def _attention_modules(self):
+        """The modules that own a paged K / V cache, in layer order."""
+        if self.model is None:
+            return []
+        if self.hybrid:
+            return self.model.attention_layers()
+        return [layer.self_attn.attn for layer in self.model.model.layers]
+
     def kv_block_bytes(self) -> int:
         m = self.cfg.model
         itemsize = torch.empty((), dtype=self.kv_dtype).element_size()
+        if self.hybrid:
+            return max(1, sum(self.block_size * a.num_kv_heads * (a.head_dim + a.v_head_dim) * itemsize
+                              for a in self.model.attention_layers()))
         return (2 * m.num_layers * self.block_size * (m.num_kv_heads // self.tp)
                 * m.head_dim * itemsize)
 
@@ -590,6 +609,10 @@ class ModelRunner:
             # same accounting as the reference (model_runner.py:140-157): budget = total *
             # utilisation - what is in use now - the activation head-room seen in warm-up
             budget = int(total * cfg.gpu_memory_utilization) - used - max(peak - current, 0)
+            if self.hybrid:
+                # no warm-up ran: keep room for a step's activations (fp32 stream + the widest
+                # projection outputs) and for the recurrent state slots
+                budget -= self._state_bytes() + cfg.max_num_batched_tokens * self._widest_row_bytes()
             num_blocks = budget // block_bytes
             if self.world_size > 1:        # every rank must agree on the block count
                 t = torch.tensor([num_blocks], dtype=torch.int64, device=self.device)
@@ -607,16 +630,43 @@ class ModelRunner:
         if num_blocks <= 0:
             raise RuntimeError("not enough device memory for a single KV-cache block")
         self.num_kv_blocks = int(num_blocks)
+        if self.hybrid:
+            return self._allocate_hybrid_caches()
         hkv = m.num_kv_heads // self.tp
         # physical order [2, layer, block, kv_head, token, d]; layers see the logical
         # [block, token, kv_head, d] view of it
         self.kv_cache = torch.zeros(2, m.num_layers, self.num_kv_blocks, hkv, self.block_size,
                                     m.head_dim, dtype=self.kv_dtype, device=self.device)
-        for i, layer in enumerate(self.model.model.layers):
-            attn = layer.self_attn.attn
+        for i, attn in enumerate(self._attention_modules()):
             attn.k_cache = self.kv_cache[0, i].permute(0, 2, 1, 3)
             attn.v_cache = self.kv_cache[1, i].permute(0, 2, 1, 3)
             attn.block_size = self.block_size
+
+    def _state_bytes(self) -> int:
+        return sum(self.num_state_slots * 4 * (d.num_heads * d.head_dim * d.v_head_dim
+                                               + max(d.taps - 1, 0) * d.conv_channels)
+                   for d in self.model.state_layers())
+
+    def _widest_row_bytes(self) -> int:
+        widest = max([p.shape[0] for p in self.model.parameters() if p.dim() == 2] + [1])
+        return 4 * (self.cfg.model.hidden_size * 4 + widest * 3)
+
+    def _allocate_hybrid_caches(self) -> None:
+        """One K and one V allocation per attention layer (their head sizes may differ from
+        layer to layer and between K and V), logical [block, token, kv head, d]; per recurrent
+        layer a fp32 state row and a convolution-tail row for every state slot."""
+        n, bs = self.num_kv_blocks, self.block_size
+        self.kv_cache = []
+        for a in self.model.attention_layers():
+            a.k_cache = torch.zeros(n, bs, a.num_kv_heads, a.head_dim, dtype=self.kv_dtype, device=self.device)
+            a.v_cache = torch.zeros(n, bs, a.num_kv_heads, a.v_head_dim, dtype=self.kv_dtype, device=self.device)
+            self.kv_cache.append((a.k_cache, a.v_cache))
+        for d in self.model.state_layers():
+            S = self.num_state_slots
+            d.state = torch.zeros(S, d.num_heads, d.head_dim, d.v_head_dim, dtype=torch.float32,
+                                  device=self.device)
+            d.conv_state = torch.zeros(S, max(d.taps - 1, 0), d.conv_channels, dtype=torch.float32,
+                                       device=self.device)
 
     # ============================================================ batch building
     def prepare_prefill(self, seqs: Seq[Sequence], num_decode: int = 0) -> Batch:
@@ -684,6 +734,8 @@ class ModelRunner:
             # (sequence numbers count from the first prompt)
             from minivllm_amd.ops import hip
             arrays["prefill_items"] = hip.prefill_work_items(lens[num_decode:], ends[num_decode:])
+        if self.hybrid:
+            self._add_hybrid_arrays(arrays, seqs, starts, ends, row, int(input_ids.size))
         self._add_filter_arrays(arrays, seqs)
         return Batch(is_prefill=True, num_seqs=B, num_tokens=int(input_ids.size),
                      max_seqlen_q=max_q, max_seqlen_k=max_k, has_prefix=has_prefix,
@@ -696,7 +748,7 @@ class ModelRunner:
         B = len(seqs)
         prev = self._decode_prev
         if prev is not None and prev[0] is seqs and self._last_tokens is not None \
-                and len(self._last_tokens) == B:
+                and len(self._last_tokens) == B and not self.hybrid:
             # the scheduler handed back the very same batch (steady-state decode: every
             # sequence grew by the token sampled last step, no block table changed)
             a = prev[1]
@@ -721,10 +773,42 @@ class ModelRunner:
                       positions=pos, slot_mapping=last_block * bs + pos % bs, context_lens=lens,
                       temperatures=np.fromiter((s.temperature for s in seqs), np.float32, B),
                       block_tables=tables)
+        if self.hybrid:
+            arrays["state_slots"] = np.fromiter((s.state_slot for s in seqs), np.int32, B)
+            if self.needs_aux_rows:
+                prev_tok = np.fromiter((s.token_ids[-2] if s.num_tokens > 1 else -1 for s in seqs),
+                                       np.int64, B)
+                arrays["aux_rows"] = self.model.aux_embedding_rows(arrays["input_ids"], prev_tok)
         self._add_filter_arrays(arrays, seqs)
         self._decode_prev = (seqs, arrays)
         return Batch(is_prefill=False, num_seqs=B, num_tokens=B, max_seqlen_q=1,
                      max_seqlen_k=int(lens.max()), max_context_len=int(lens.max()), arrays=arrays)
+
+    def _add_hybrid_arrays(self, arrays: dict, seqs: Seq[Sequence], starts, ends, row, padded: int) -> None:
+        """What models with recurrent state or a context-hashed embedding need besides the
+        dense arrays: each sequence's state slot, the sequence of each row (-1: padding) and the
+        auxiliary embedding row of each token (from the token before it, which for a row at
+        the start of a portion is the sequence's own earlier token)."""
+        total = int(row.size)
+        arrays["state_slots"] = np.fromiter((s.state_slot for s in seqs), np.int32, len(seqs))
+        rs = np.full(padded, -1, np.int32)
+        rs[:total] = row
+        arrays["row_seq"] = rs
+        if self.needs_aux_rows:
+            prev = np.empty(total, np.int64)
+            at = 0
+            for s, lo, hi in zip(seqs, starts.tolist(), ends.tolist()):
+                n = hi - lo
+                if lo > 0:
+                    prev[at:at + n] = s.token_array(lo - 1, hi - 1) if n > 1 else s.token_ids[lo - 1]
+                else:
+                    prev[at] = -1
+                    if n > 1:
+                        prev[at + 1:at + n] = s.token_array(0, hi - 1)
+                at += n
+            aux = np.zeros(padded, np.int32)
+            aux[:total] = self.model.aux_embedding_rows(arrays["input_ids"][:total], prev)
+            arrays["aux_rows"] = aux
 
     @staticmethod
     def _add_filter_arrays(arrays: dict, seqs: Seq[Sequence]) -> None:
@@ -769,7 +853,7 @@ class ModelRunner:
             # starts: the tables every rank derives the next step from must hold it
             batch.arrays["block_tables"] = _pad_block_tables([s.block_table for s in seqs])
             batch.tables_unchanged = False
-        if is_prefill and next_prefill is not None and num_decode == 0:
+        if is_prefill and next_prefill is not None and num_decode == 0 and not self.hybrid:
             return self._run_prefill_with_lookahead(batch, next_prefill, self._PG_KEY_UNSET)
         if self.world_size > 1 and self.rank == 0:
             self.channel.send("run_batch", batch.scalars(), batch.arrays)
@@ -782,6 +866,49 @@ class ModelRunner:
                 self._last_tokens = out
                 return out
             return self.execute(batch)
+
+    # ----------------------------------------------------------------- scoring
+    def score(self, seqs: Seq[Sequence], is_prefill: bool, num_decode: int = 0,
+              want: Optional[Dict[int, List[int]]] = None) -> Dict[int, torch.Tensor]:
+        """One step over given tokens whose result is logits, not samples.  ``seqs`` /
+        ``is_prefill`` / ``num_decode`` as for ``run`` (what ``Scheduler.schedule_given``
+        returns); ``want``: seq_id -> offsets inside the sequence's portion of this step whose
+        logits are asked for.  Runs the same batch preparation, upload, forward (decode graphs
+        included) as ``run``; returns seq_id -> fp32 CPU tensor [asked, vocab]."""
+        assert self._spec is None and self._pf_spec is None and self.world_size == 1
+        want = want or {}
+        V = self.cfg.model.vocab_size
+        if is_prefill:
+            self._decode_prev = None
+            batch = self.prepare_prefill(seqs, num_decode)
+            n = len(seqs)
+            inner = list(seqs[n - num_decode:]) + list(seqs[:n - num_decode]) if num_decode else list(seqs)
+            cu = batch.arrays["cu_seqlens_q"]
+            rows, owner = [], []
+            for i, s in enumerate(inner):
+                for off in want.get(s.seq_id, ()):
+                    if not 0 <= off < cu[i + 1] - cu[i]:
+                        raise ValueError("asked for logits outside the sequence's portion")
+                    rows.append(int(cu[i]) + off)
+                    owner.append(s.seq_id)
+            if not rows:                       # nothing asked: still one row, the head is cheap
+                rows, owner = [0], [None]
+            batch.arrays["logit_rows"] = np.asarray(rows, np.int32)
+        else:
+            batch = self.prepare_decode(seqs)
+            owner = [s.seq_id if want.get(s.seq_id) else None for s in seqs]
+        self.step_counter += 1
+        batch.step = self.step_counter
+        with torch.inference_mode(), trace_range("score_step"):
+            self.execute(batch)
+            logits = self._last_step_logits[:len(owner), :V].float().cpu()
+        self._last_tokens = None
+        self._decode_prev = None
+        out: Dict[int, list] = {}
+        for r, sid in enumerate(owner):
+            if sid is not None:
+                out.setdefault(sid, []).append(logits[r])
+        return {sid: torch.stack(v) for sid, v in out.items()}
 
     # --------------------------------------------------- prefill launched one step ahead
     # Between two prefill steps the GPU otherwise idles while the host reads the samples back,
@@ -801,7 +928,7 @@ class ModelRunner:
     _PG_KEY_UNSET = object()
 
     def _prefill_can_go_ahead(self, b: Batch, key) -> bool:
-        if not self.cfg.prefill_prelaunch or "top_k" in b.arrays or b.num_decode_seqs:
+        if not self.cfg.prefill_prelaunch or "top_k" in b.arrays or b.num_decode_seqs or self.hybrid:
             return False
         if os.environ.get("MINIVLLM_NO_PRELAUNCH") == "1":
             return False
@@ -896,6 +1023,8 @@ class ModelRunner:
     def _can_prelaunch(self, b: Batch) -> bool:
         if b.is_prefill or not self.cfg.decode_prelaunch or "top_k" in b.arrays:
             return False
+        if self.needs_aux_rows:
+            return False     # the next step's embedding rows depend on the token sampled now
         if os.environ.get("MINIVLLM_NO_PRELAUNCH") == "1":
             return False
         if self.on_gpu and self._graph_bucket(b.num_seqs) is None:
@@ -922,7 +1051,8 @@ class ModelRunner:
         t = self._decode_tensors(B)
         set_context(False, slot_mapping=t["slot_mapping"], context_lens=t["context_lens"],
                     block_tables=t["block_tables"], positions=t["positions"],
-                    max_context_len=b.max_context_len, num_seqs=B, positions_in_context=True)
+                    max_context_len=b.max_context_len, num_seqs=B, positions_in_context=True,
+                    state_slots=t["state_slots"], aux_rows=t["aux_rows"])
         tokens = self._forward_and_sample(t)
         reset_context()
         return tokens
@@ -1013,6 +1143,10 @@ class ModelRunner:
                         ("cu_seqlens_q", B + 1), ("cu_seqlens_k", B + 1), ("temperatures", B),
                         ("misc", 4), ("context_lens", b.num_decode_seqs),
                         ("prefill_items", a["prefill_items"].size if "prefill_items" in a else 0),
+                        ("aux_rows", a["aux_rows"].size if "aux_rows" in a else 0),
+                        ("row_seq", a["row_seq"].size if "row_seq" in a else 0),
+                        ("state_slots", a["state_slots"].size if "state_slots" in a else 0),
+                        ("logit_rows", a["logit_rows"].size if "logit_rows" in a else 0),
                         ("block_tables", B * MB)):
             layout[name] = (off, n)
             off += al(n)
@@ -1035,6 +1169,10 @@ class ModelRunner:
                     temperatures=v("temperatures").view(torch.float32),
                     step=v("misc"), context_lens=v("context_lens"),
                     prefill_items=v("prefill_items") if "prefill_items" in a else None,
+                    aux_rows=v("aux_rows") if "aux_rows" in a else None,
+                    row_seq=v("row_seq") if "row_seq" in a else None,
+                    state_slots=v("state_slots") if "state_slots" in a else None,
+                    logit_rows=v("logit_rows") if "logit_rows" in a else None,
                     positions_in_context=True,
                     block_tables=v("block_tables").view(B, MB))
 
@@ -1056,6 +1194,10 @@ class ModelRunner:
         put("slot_mapping", a["slot_mapping"], -1)
         put("context_lens", a["context_lens"], 0)
         put("temperatures", a["temperatures"].astype(np.float32).view(np.int32), 0)
+        if "state_slots" in a:
+            put("state_slots", a["state_slots"], -1)
+        if "aux_rows" in a:
+            put("aux_rows", a["aux_rows"], 0)
         host[self._dec_off["misc"][0]] = b.step
         # Which table rows a staging block already holds is tracked by a counter, never by the
         # identity of the numpy array: a freed array's address is handed to the next one, and a
@@ -1109,6 +1251,8 @@ class ModelRunner:
                     context_lens=self._dec_view(d, "context_lens", n),
                     temperatures=self._dec_view(d, "temperatures", n).view(torch.float32),
                     step=self._dec_view(d, "misc"),
+                    aux_rows=self._dec_view(d, "aux_rows", n) if self.needs_aux_rows else None,
+                    state_slots=self._dec_view(d, "state_slots", n) if self.num_state_slots else None,
                     block_tables=self._dec_view(d, "block_tables", n * MB).view(n, MB))
 
     # -------------------------------------------------------------- execute
@@ -1127,8 +1271,9 @@ class ModelRunner:
                     context_lens=t["context_lens"] if b.num_decode_seqs else None,
                     max_context_len=b.max_context_len, total_k_tokens=b.num_prefill_k_tokens,
                     prefill_items=None if warmup else t["prefill_items"],
-                    positions_in_context=True)
-        tokens = self._forward_and_sample(t)
+                    positions_in_context=True, state_slots=t["state_slots"],
+                    aux_rows=t["aux_rows"], row_seq=t["row_seq"], logit_rows=t["logit_rows"])
+        tokens = self._forward_and_sample(t, score_only=t["logit_rows"] is not None)
         return tokens, self._last_logits
 
     def execute(self, b: Batch, warmup: bool = False, pg_key=_PG_KEY_UNSET) -> Optional[List[int]]:
@@ -1153,7 +1298,8 @@ class ModelRunner:
                 set_context(False, slot_mapping=t["slot_mapping"], context_lens=t["context_lens"],
                             block_tables=t["block_tables"], positions=t["positions"],
                             max_context_len=b.max_context_len, num_seqs=B,
-                            positions_in_context=True)
+                            positions_in_context=True, state_slots=t["state_slots"],
+                            aux_rows=t["aux_rows"])
                 tokens = self._forward_and_sample(t)
                 logits = self._last_logits
         reset_context()
@@ -1183,17 +1329,26 @@ class ModelRunner:
                 return s
         return None
 
-    def _forward_and_sample(self, t: dict) -> Optional[torch.Tensor]:
+    def _forward_and_sample(self, t: dict, score_only: bool = False) -> Optional[torch.Tensor]:
         hidden = self.model(t["input_ids"], t["positions"])
+        if score_only:
+            # a scoring step: the logits of the asked rows are the result, nothing is drawn
+            self._last_logits = self.model.lm_head.local_logits(hidden)
+            return None
         return self._sample(hidden, t["temperatures"], t["step"])
 
     def _sample(self, hidden: torch.Tensor, temperatures: torch.Tensor,
                 step: torch.Tensor) -> Optional[torch.Tensor]:
         if self.on_gpu:
-            from minivllm_amd.ops import hip
             head = self.model.lm_head
             logits = head.local_logits(hidden)
             self._last_logits = logits
+            if logits.dtype != torch.float32:
+                from minivllm_amd.ops import hip
+            if logits.dtype == torch.float32:
+                # the sampling kernel takes 16-bit logits; a 32-bit engine draws with the
+                # PyTorch sampler
+                return self.sampler(logits[..., :head.num_embeddings], temperatures).to(torch.int32)
             vals, idx = hip.sample_local(logits, temperatures, self.cfg.seed, step,
                                          vocab_offset=head.vocab_start,
                                          valid_vocab=head.num_embeddings)
@@ -1316,6 +1471,8 @@ class ModelRunner:
         host[o:o + n] = -1
         o, n = self._dec_off["block_tables"]
         host[o:o + n] = -1
+        o, n = self._dec_off["state_slots"]
+        host[o:o + n] = -1
         self._dec_dev.copy_(self._dec_host)
         for bs in reversed(self._graph_sizes):
             t = self._decode_tensors(bs)
@@ -1324,7 +1481,8 @@ class ModelRunner:
                 set_context(False, slot_mapping=t["slot_mapping"], context_lens=t["context_lens"],
                             block_tables=t["block_tables"], positions=t["positions"],
                             max_context_len=self.cfg.max_model_length, num_seqs=bs,
-                            positions_in_context=True)
+                            positions_in_context=True, state_slots=t["state_slots"],
+                            aux_rows=t["aux_rows"])
                 out = self._forward_and_sample(t)
                 reset_context()
                 return out

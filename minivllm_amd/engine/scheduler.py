@@ -38,7 +38,8 @@ class Scheduler:
                  max_cached_blocks: int, block_size: int, eos: int,
                  max_model_length: Optional[int] = None, enable_chunked_prefill: bool = True,
                  min_prefill_tokens: int = 0, max_prefill_delay_s: float = 0.0,
-                 enable_mixed_batches: bool = False, ahead_over_block_edges: bool = True):
+                 enable_mixed_batches: bool = False, ahead_over_block_edges: bool = True,
+                 num_state_slots: int = 0, prefix_caching: bool = True):
         self.enable_chunked_prefill = enable_chunked_prefill
         # decode steps launched ahead may cross KV-block edges (blocks allocated ahead, block
         # hashes published when the step is collected) and go on while requests wait that cannot
@@ -62,7 +63,12 @@ class Scheduler:
         self.num_mixed_steps = 0
         # admitted (blocks allocated) but not yet completely prefetched, oldest first
         self.prefilling: Deque[Sequence] = deque()
-        self.block_manager = make_block_manager(max_cached_blocks, block_size)
+        self.block_manager = make_block_manager(max_cached_blocks, block_size,
+                                                prefix_caching=prefix_caching)
+        # models with per-sequence recurrent state: a slot is taken with a sequence's KV blocks
+        # and given back with them (admission, preemption, finish, abort)
+        from .state_pool import StateSlotPool
+        self.state_pool = StateSlotPool(num_state_slots) if num_state_slots else None
         self.max_num_sequences = max_num_sequences
         self.max_num_batched_tokens = max_num_batched_tokens
         self.max_model_length = max_model_length
@@ -197,8 +203,10 @@ class Scheduler:
                 break
             if len(self.running) >= self.max_num_sequences:
                 break
+            if self.state_pool is not None and not self.state_pool.num_free:
+                break
             self.waiting.popleft()
-            bm.allocate(seq)
+            self._allocate(seq)
             seq.status = SequenceStatus.RUNNING
             todo = len(seq) - seq.num_cached_tokens
             take = todo
@@ -358,10 +366,21 @@ class Scheduler:
             return age < self.max_prefill_delay_s
         return False
 
+    def _allocate(self, seq: Sequence) -> None:
+        self.block_manager.allocate(seq)
+        if self.state_pool is not None:
+            seq.state_slot = self.state_pool.allocate()
+
+    def _deallocate(self, seq: Sequence, num_valid_tokens: Optional[int] = None) -> None:
+        self.block_manager.deallocate(seq, num_valid_tokens)
+        if self.state_pool is not None and seq.state_slot >= 0:
+            self.state_pool.release(seq.state_slot)
+            seq.state_slot = -1
+
     def preempt(self, seq: Sequence) -> None:
         self._decode_batch = None
         seq.prefill_end = None
-        self.block_manager.deallocate(seq)
+        self._deallocate(seq)
         seq.status = SequenceStatus.WAITING
         self.waiting.appendleft(seq)
         self.num_preemptions += 1
@@ -393,10 +412,70 @@ class Scheduler:
                 valid = seq.num_tokens - 1       # the newest token's KV slot may be unwritten
             else:
                 valid = None
-            self.block_manager.deallocate(seq, valid)
+            self._deallocate(seq, valid)
         seq.prefill_end = None
         seq.status = SequenceStatus.FINISHED
         return True
+
+    # ------------------------------------------------- steps whose make-up is given
+    # Scoring a given text (no sampling: every token is known) and replaying a recorded
+    # schedule: the caller says which sequences take part in the step and how many of their
+    # next tokens each one computes; admission, KV blocks and state slots are still this
+    # scheduler's business.  A sequence may sit a step out and may gain tokens between steps
+    # (``Sequence.extend_tokens``).
+    def schedule_given(self, portions: List[Tuple[Sequence, int]]) -> Tuple[List[Sequence], bool, int]:
+        """``portions``: (sequence, number of its next tokens to compute).  Admits the
+        sequences that are still waiting, brings the others' block tables up to their length,
+        and returns (sequences in step order, is_prefill, number of trailing decode riders) as
+        ``schedule`` + ``last_num_decode`` would: a step of single next tokens of running
+        sequences only is a decode step; otherwise single-token entries of sequences that have
+        nothing else outstanding ride along a prefill-form step.  Raises when blocks, slots or
+        sequence budget do not suffice (nothing is preempted for a given schedule)."""
+        bm = self.block_manager
+        self._decode_batch = None
+        if len(portions) > self.max_num_sequences:
+            raise RuntimeError("more sequences in one step than max_num_sequences")
+        prompts: List[Sequence] = []
+        riders: List[Sequence] = []
+        for seq, n in portions:
+            if n <= 0:
+                raise ValueError("a portion computes at least one token")
+            if seq.status == SequenceStatus.WAITING:
+                if not bm.can_allocate(seq) or (self.state_pool is not None and not self.state_pool.num_free) \
+                        or len(self.running) >= self.max_num_sequences:
+                    raise RuntimeError("no room to admit a sequence of the given step")
+                self.waiting.remove(seq)
+                self._allocate(seq)
+                seq.status = SequenceStatus.RUNNING
+                self.running.append(seq)
+            elif seq.status != SequenceStatus.RUNNING:
+                raise ValueError("a finished sequence cannot take part in a step")
+            else:
+                if not bm.can_grow(seq):
+                    raise RuntimeError("out of KV blocks for the given step")
+                bm.grow(seq)
+            end = seq.num_cached_tokens + n
+            if end > seq.num_tokens:
+                raise ValueError("a portion reaches beyond the tokens the sequence has")
+            seq.prefill_end = end
+            rider = n == 1 and seq.num_cached_tokens > 0 and end == seq.num_tokens
+            (riders if rider else prompts).append(seq)
+        if not prompts:
+            for s in riders:
+                s.prefill_end = None
+            return riders, False, 0
+        self.last_num_decode = len(riders)
+        return prompts + riders, True, len(riders)
+
+    def advance_given(self, seqs: List[Sequence]) -> None:
+        """After a given step ran: what it computed is in the cache (and the state)."""
+        for seq in seqs:
+            seq.num_cached_tokens = seq.num_tokens if seq.prefill_end is None else seq.prefill_end
+            seq.prefill_end = None
+
+    def release(self, seq: Sequence) -> None:
+        """A sequence of a given schedule has ended: its blocks and slot go back."""
+        self.abort(seq)
 
     # ---------------------------------------------------------- postprocess
     def postprocess(self, seqs: List[Sequence], token_ids: List[int]) -> List[Sequence]:
@@ -418,7 +497,7 @@ class Scheduler:
                        and seq.num_tokens >= self.max_model_length)
             if hit_eos or hit_len or hit_ctx:
                 seq.status = SequenceStatus.FINISHED
-                self.block_manager.deallocate(seq)
+                self._deallocate(seq)
                 finished.append(seq)
         if finished:
             self._decode_batch = None

@@ -35,6 +35,8 @@ class Sequence:
     stop_token_ids: frozenset = frozenset()
     top_k: int = 0
     top_p: float = 1.0
+    # slot of the sequence's recurrent state (models that have one), -1 = none
+    state_slot: int = -1
 
     def __init__(self, token_ids: List[int], sampling_params: Optional[SamplingParams] = None,
                  block_size: Optional[int] = None):
@@ -118,6 +120,12 @@ class Sequence:
         """Tokens the scheduled prefill step computes for this sequence."""
         end = self.num_tokens if self.prefill_end is None else self.prefill_end
         return end - self.num_cached_tokens
+
+    def extend_tokens(self, token_ids) -> None:
+        """Append given tokens (the continuation of a text that is being scored, as opposed to
+        tokens the engine sampled)."""
+        for t in token_ids:
+            self.append_token(int(t))
 
     def append_token(self, token_id: int) -> None:
         self.token_ids.append(token_id)
