@@ -2,6 +2,8 @@
 
 * ``_hip_kernels.so``  - every gfx950 kernel under ``csrc/*.hip`` (hipcc, one object per
   source, C ABI launchers that take raw device pointers and a ``hipStream_t``).
+* ``_hip_hybrid.so``   - the kernels of hybrid decoders under ``csrc/hybrid/*.hip`` (a library of
+  its own, so that a program serving only such a model builds, and loads, nothing else).
 * ``_host_core.so``    - host-side C++ (csrc/host/*.cpp), no GPU code.
 
 ``python -m minivllm_amd.build`` builds whatever is out of date; ``--force`` rebuilds all.
@@ -22,6 +24,8 @@ CSRC = os.path.join(HERE, "csrc")
 BUILD = os.path.join(HERE, "csrc", "build")
 HIP_LIB = os.path.join(HERE, "_hip_kernels.so")
 HOST_LIB = os.path.join(HERE, "_host_core.so")
+# further kernel libraries: name -> (source folder under csrc, library file)
+GROUPS = {"hybrid": ("hybrid", os.path.join(HERE, "_hip_hybrid.so"))}
 ARCH = "gfx950"
 
 
@@ -55,18 +59,30 @@ def _file_flags(src: str) -> list:
 
 
 def build_hip(force: bool = False, verbose: bool = True) -> str:
-    srcs = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
-    hdrs = sorted(glob.glob(os.path.join(CSRC, "*.h")))
+    return _build_hip_lib(CSRC, HIP_LIB, "", force, verbose)
+
+
+def build_hip_group(name: str, force: bool = False, verbose: bool = True) -> str:
+    folder, lib = GROUPS[name]
+    return _build_hip_lib(os.path.join(CSRC, folder), lib, name + "_", force, verbose)
+
+
+def _build_hip_lib(src_dir: str, HIP_LIB: str, prefix: str, force: bool, verbose: bool) -> str:
+    srcs = sorted(glob.glob(os.path.join(src_dir, "*.hip")))
+    hdrs = sorted(glob.glob(os.path.join(src_dir, "*.h")))
     if not force and _newer(HIP_LIB, srcs + hdrs):
         return HIP_LIB                       # library is newer than every source: keep it
     os.makedirs(BUILD, exist_ok=True)
     hipcc = _hipcc()
+    # packed fp32 instructions are never generated (-packed-fp32-ops: the compiler otherwise
+    # forms them from ordinary float code)
     flags = [f"--offload-arch={ARCH}", "-O3", "-fPIC", "-std=c++17", "-Wall",
-             "-Wno-unused-function", "-Wno-unused-variable"]
+             "-Wno-unused-function", "-Wno-unused-variable",
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
     jobs = []
     objs = []
     for s in srcs:
-        o = os.path.join(BUILD, os.path.basename(s) + ".o")
+        o = os.path.join(BUILD, prefix + os.path.basename(s) + ".o")
         objs.append(o)
         if force or not _newer(o, [s] + hdrs):
             jobs.append([hipcc] + flags + _file_flags(s) + ["-c", s, "-o", o])
@@ -76,7 +92,9 @@ def build_hip(force: bool = False, verbose: bool = True) -> str:
         with ThreadPoolExecutor(max_workers=min(len(jobs), int(os.environ.get("MAX_JOBS", 6)))) as ex:
             list(ex.map(_run, jobs))
     if jobs or not _newer(HIP_LIB, objs):
-        _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", HIP_LIB] + objs)
+        tmp = f"{HIP_LIB}.{os.getpid()}.tmp"         # (two first calls at once: whole files only)
+        _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", tmp] + objs)
+        os.replace(tmp, HIP_LIB)
         if verbose:
             print(f"[build] linked {HIP_LIB}", flush=True)
     return HIP_LIB
@@ -97,6 +115,8 @@ def build_host(force: bool = False, verbose: bool = True) -> str:
 
 def build_all(force: bool = False, verbose: bool = True) -> None:
     build_hip(force, verbose)
+    for name in GROUPS:
+        build_hip_group(name, force, verbose)
     build_host(force, verbose)
 
 

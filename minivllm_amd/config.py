@@ -255,6 +255,9 @@ class EngineConfig:
     # Generated tokens are meaningless (partial sums are never completed).  0 = off.
     tp_shard: int = 0
     tp_shard_rank: int = 0
+    # the engine only scores given text (LLMEngine.score_step): every step ends at the logits
+    # and draws nothing, decode graphs are captured without the sampler
+    score_only: bool = False
     # number of engine replicas behind engine.dp_engine.DataParallelEngine (1 = none)
     data_parallel_size: int = 1
 

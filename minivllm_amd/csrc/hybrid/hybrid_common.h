@@ -1,0 +1,73 @@
+// Helpers shared by the kernels of hybrid decoders (fp32 residual stream, zero-centred norms,
+// attention with a sink, gated delta rule, grouped expert routing).  Activations are bfloat16
+// or float (template parameter), everything a norm, a softmax or a recurrence touches is fp32.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace hyb {
+
+constexpr int kWave = 64;
+
+struct bf16_t { uint16_t v; };
+
+template <typename T> __device__ __forceinline__ float ld(const T* p);
+template <> __device__ __forceinline__ float ld<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float ld<bf16_t>(const bf16_t* p) {
+    return __uint_as_float(((uint32_t)p->v) << 16);
+}
+template <typename T> __device__ __forceinline__ void st(T* p, float f);
+template <> __device__ __forceinline__ void st<float>(float* p, float f) { *p = f; }
+template <> __device__ __forceinline__ void st<bf16_t>(bf16_t* p, float f) {
+    __bf16 b = (__bf16)f;                          // round to nearest even
+    p->v = __builtin_bit_cast(uint16_t, b);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+    return v;
+}
+
+// sum over a workgroup of up to 1024 threads; `red` holds 16 floats of LDS; every thread gets it
+__device__ __forceinline__ float block_sum(float v, float* red) {
+    v = wave_sum(v);
+    const int w = threadIdx.x / kWave, nw = (blockDim.x + kWave - 1) / kWave;
+    __syncthreads();
+    if ((threadIdx.x & (kWave - 1)) == 0) red[w] = v;
+    __syncthreads();
+    float s = 0.f;
+    for (int i = 0; i < nw; ++i) s += red[i];
+    return s;
+}
+__device__ __forceinline__ float block_max(float v, float* red) {
+    v = wave_max(v);
+    const int w = threadIdx.x / kWave, nw = (blockDim.x + kWave - 1) / kWave;
+    __syncthreads();
+    if ((threadIdx.x & (kWave - 1)) == 0) red[w] = v;
+    __syncthreads();
+    float s = red[0];
+    for (int i = 1; i < nw; ++i) s = fmaxf(s, red[i]);
+    return s;
+}
+
+__device__ __forceinline__ float sigmoidf_(float z) { return 1.f / (1.f + expf(-z)); }
+__device__ __forceinline__ float siluf_(float z) { return z / (1.f + expf(-z)); }
+__device__ __forceinline__ float softplusf_(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+__device__ __forceinline__ float gelu_erf(float z) { return 0.5f * z * (1.f + erff(z * 0.70710678118654752f)); }
+
+#define HYB_DISPATCH(dt, ...)                                         \
+    do {                                                              \
+        if ((dt) == 0) { using T = hyb::bf16_t; __VA_ARGS__; }        \
+        else if ((dt) == 2) { using T = float; __VA_ARGS__; }         \
+        else return 1;                                                \
+    } while (0)
+
+#define HYB_LAUNCH_OK() (hipGetLastError() == hipSuccess ? 0 : 2)
+
+}  // namespace hyb

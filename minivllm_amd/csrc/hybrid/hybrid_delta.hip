@@ -1,0 +1,227 @@
+// Gated delta rule: preparation of a step's tokens (short causal convolution + silu on q / k / v,
+// unit vectors, beta and decay) and the recurrence itself, for prefill portions and single
+// decode tokens alike.  Everything here is fp32 except the projection outputs it reads.
+//
+// Sequence layout: `cu_q` [B+1] rows of each sequence (null: row b is sequence b), `positions`
+// (a sequence's first row holds the position its portion starts at; 0 = start from zeros),
+// `slots` [B] state slot per sequence (< 0: unused row of a padded batch), `row_seq` [T] the
+// sequence of each row in prefill form (< 0: no sequence).
+#include "hybrid_common.h"
+
+using namespace hyb;
+
+constexpr int MAX_TAPS = 8;
+
+// One workgroup per token row.  proj row = [q (G*D) | k (G*D) | v (H*E) | gate | b (H) | a (H)];
+// the three convolved blocks are contiguous at the row's start (C = 2GD + HE channels).
+// conv_w [C, taps] (q, k, v rows stacked), conv_state [slots, taps-1, C].
+template <typename T>
+__global__ void delta_prepare_kernel(const T* __restrict__ proj, long row_stride, int b_off,
+                                     int a_off, const float* __restrict__ conv_w, int taps,
+                                     const float* __restrict__ a_log,
+                                     const float* __restrict__ dt_bias,
+                                     const float* __restrict__ conv_state,
+                                     const int* __restrict__ cu_q, const int* __restrict__ positions,
+                                     const int* __restrict__ slots, const int* __restrict__ row_seq,
+                                     float* __restrict__ qn, float* __restrict__ kn,
+                                     float* __restrict__ vv, float* __restrict__ beta,
+                                     float* __restrict__ decay, int H, int G, int D, int E) {
+    extern __shared__ float y[];                     // [2GD] convolved + silu q, k
+    const long t = blockIdx.x;
+    const int b = row_seq ? row_seq[t] : (int)t;
+    if (b < 0) return;
+    const int slot = slots[b];
+    if (slot < 0) return;
+    const long first = cu_q ? cu_q[b] : t;           // the sequence's first row in this step
+    const int i = (int)(t - first);                  // index inside the portion
+    const bool has_past = positions[first] > 0;
+    const int C = 2 * G * D + H * E, GD = G * D;
+    const float* tail = conv_state + (long)slot * (taps - 1) * C;
+    for (int c = threadIdx.x; c < C; c += blockDim.x) {
+        float acc = 0.f;
+        for (int j = 0; j < taps; ++j) {             // tap j reads the input `taps-1-j` tokens back
+            const int back = taps - 1 - j;
+            float x;
+            if (i - back >= 0) x = ld(proj + (t - back) * row_stride + c);
+            else x = has_past ? tail[(long)(taps - 1 + i - back) * C + c] : 0.f;
+            acc += x * conv_w[(long)c * taps + j];
+        }
+        acc = siluf_(acc);
+        if (c < 2 * GD) y[c] = acc;
+        else vv[t * (long)(H * E) + (c - 2 * GD)] = acc;
+    }
+    __syncthreads();
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1), nw = blockDim.x / kWave;
+    for (int hd = wave; hd < 2 * G; hd += nw) {      // heads of q (0..G-1) then of k
+        const float* src = y + hd * D;
+        float s = 0.f;
+        for (int d = lane; d < D; d += kWave) s += src[d] * src[d];
+        float r = rsqrtf(wave_sum(s) + 1e-6f);
+        float* dst;
+        if (hd < G) { r *= rsqrtf((float)D); dst = qn + (t * G + hd) * (long)D; }
+        else dst = kn + (t * G + hd - G) * (long)D;
+        for (int d = lane; d < D; d += kWave) dst[d] = src[d] * r;
+    }
+    for (int h = threadIdx.x; h < H; h += blockDim.x) {
+        beta[t * H + h] = sigmoidf_(ld(proj + t * row_stride + b_off + h));
+        const float z = ld(proj + t * row_stride + a_off + h) + dt_bias[h];
+        decay[t * H + h] = expf(-expf(a_log[h]) * softplusf_(z));
+    }
+}
+
+// One workgroup per sequence: the convolution inputs of the portion's last taps-1 tokens become
+// the slot's tail (older entries shift when the portion is shorter).  Runs after delta_prepare.
+template <typename T>
+__global__ void delta_conv_tail_kernel(const T* __restrict__ proj, long row_stride, int taps,
+                                       float* __restrict__ conv_state,
+                                       const int* __restrict__ cu_q,
+                                       const int* __restrict__ positions,
+                                       const int* __restrict__ slots, int C) {
+    const int b = blockIdx.x;
+    const int slot = slots[b];
+    if (slot < 0 || taps <= 1) return;
+    const long first = cu_q ? cu_q[b] : b;
+    const int n = cu_q ? cu_q[b + 1] - cu_q[b] : 1;
+    if (n <= 0) return;
+    const bool has_past = positions[first] > 0;
+    float* tail = conv_state + (long)slot * (taps - 1) * C;
+    for (int c = threadIdx.x; c < C; c += blockDim.x) {
+        float nv[MAX_TAPS];
+#pragma unroll
+        for (int j = 0; j < MAX_TAPS - 1; ++j) {
+            if (j < taps - 1) {
+                const int i = n - (taps - 1) + j;    // index inside the portion, may be negative
+                if (i >= 0) nv[j] = ld(proj + (first + i) * row_stride + c);
+                else nv[j] = has_past ? tail[(long)(taps - 1 + i) * C + c] : 0.f;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < MAX_TAPS - 1; ++j)
+            if (j < taps - 1) tail[(long)j * C + c] = nv[j];
+    }
+}
+
+// The recurrence.  A state column S[:, e] evolves independently of the others:
+//   u_e = beta (v_e - g sum_d S[d,e] k_d);  S[d,e] <- g S[d,e] + k_d u_e;  o_e = sum_d S[d,e] q_d
+// so a column is owned by 4 neighbouring lanes, lane r holding d in [r*NR, (r+1)*NR) in
+// registers (D <= 4*NR, missing d padded with zeros).  Workgroup = 64 columns of one (sequence,
+// head); tokens are walked in order with the next token's k / q loads issued ahead.
+template <int NR>
+__global__ void __launch_bounds__(256)
+delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
+                  const float* __restrict__ vv, const float* __restrict__ beta,
+                  const float* __restrict__ decay, float* __restrict__ state,
+                  const int* __restrict__ cu_q, const int* __restrict__ positions,
+                  const int* __restrict__ slots, float* __restrict__ o, int H, int G, int D, int E) {
+    const int b = blockIdx.x, h = blockIdx.y;
+    const int slot = slots[b];
+    if (slot < 0) return;
+    const long first = cu_q ? cu_q[b] : b;
+    const int n = cu_q ? cu_q[b + 1] - cu_q[b] : 1;
+    if (n <= 0) return;
+    const int r = threadIdx.x & 3;
+    const int e = blockIdx.z * 64 + (threadIdx.x >> 2);
+    const bool col = e < E;
+    const int g = h / (H / G);
+    const int d0 = r * NR;
+    float S[NR];
+    float* sp = state + (((long)slot * H + h) * D) * E + e;
+    const bool has_past = positions[first] > 0;
+#pragma unroll
+    for (int i = 0; i < NR; ++i)
+        S[i] = (has_past && col && d0 + i < D) ? sp[(long)(d0 + i) * E] : 0.f;
+    float kc[NR], qc[NR];
+    auto load_kq = [&](long t, float* kk, float* qq) {
+        const float* kp = kn + (t * G + g) * (long)D + d0;
+        const float* qp = qn + (t * G + g) * (long)D + d0;
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+            const bool ok = d0 + i < D;
+            kk[i] = ok ? kp[i] : 0.f;
+            qq[i] = ok ? qp[i] : 0.f;
+        }
+    };
+    load_kq(first, kc, qc);
+    for (int s = 0; s < n; ++s) {
+        const long t = first + s;
+        float kx[NR], qx[NR];
+        if (s + 1 < n) load_kq(t + 1, kx, qx);
+        const float gd = decay[t * H + h], bt = beta[t * H + h];
+        const float ve = col ? vv[(t * H + h) * (long)E + e] : 0.f;
+        float dot = 0.f;
+#pragma unroll
+        for (int i = 0; i < NR; ++i) dot += S[i] * kc[i];
+        dot += __shfl_xor(dot, 1, kWave);
+        dot += __shfl_xor(dot, 2, kWave);
+        const float u = bt * (ve - gd * dot);
+        float out = 0.f;
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+            S[i] = gd * S[i] + kc[i] * u;
+            out += S[i] * qc[i];
+        }
+        out += __shfl_xor(out, 1, kWave);
+        out += __shfl_xor(out, 2, kWave);
+        if (col && r == 0) o[(t * H + h) * (long)E + e] = out;
+        if (s + 1 < n) {
+#pragma unroll
+            for (int i = 0; i < NR; ++i) { kc[i] = kx[i]; qc[i] = qx[i]; }
+        }
+    }
+    if (col) {
+#pragma unroll
+        for (int i = 0; i < NR; ++i)
+            if (d0 + i < D) sp[(long)(d0 + i) * E] = S[i];
+    }
+}
+
+extern "C" {
+
+int hyb_delta_prepare(const void* proj, long row_stride, int b_off, int a_off, const void* conv_w,
+                      int taps, const void* a_log, const void* dt_bias, void* conv_state,
+                      const void* cu_q, const void* positions, const void* slots,
+                      const void* row_seq, void* qn, void* kn, void* vv, void* beta, void* decay,
+                      long T_, int B, int H, int G, int D, int E, int dt, hipStream_t s) {
+    if (T_ <= 0) return 0;
+    if (taps < 1 || taps > MAX_TAPS || H % G) return 1;
+    const int C = 2 * G * D + H * E;
+    const size_t lds = 2 * (size_t)G * D * sizeof(float);
+    if (lds > 64 * 1024) return 1;
+    HYB_DISPATCH(dt, hipLaunchKernelGGL(delta_prepare_kernel<T>, dim3(T_), dim3(256), lds, s,
+                                        (const T*)proj, row_stride, b_off, a_off,
+                                        (const float*)conv_w, taps, (const float*)a_log,
+                                        (const float*)dt_bias, (const float*)conv_state,
+                                        (const int*)cu_q, (const int*)positions, (const int*)slots,
+                                        (const int*)row_seq, (float*)qn, (float*)kn, (float*)vv,
+                                        (float*)beta, (float*)decay, H, G, D, E));
+    if (hipGetLastError() != hipSuccess) return 2;
+    if (taps > 1) {
+        HYB_DISPATCH(dt, hipLaunchKernelGGL(delta_conv_tail_kernel<T>, dim3(B), dim3(256), 0, s,
+                                            (const T*)proj, row_stride, taps, (float*)conv_state,
+                                            (const int*)cu_q, (const int*)positions,
+                                            (const int*)slots, C));
+    }
+    return HYB_LAUNCH_OK();
+}
+
+int hyb_delta_scan(const void* qn, const void* kn, const void* vv, const void* beta,
+                   const void* decay, void* state, const void* cu_q, const void* positions,
+                   const void* slots, void* o, int B, int H, int G, int D, int E, hipStream_t s) {
+    if (B <= 0) return 0;
+    if (H % G || D > 512) return 1;
+    const dim3 grid(B, H, (E + 63) / 64), block(256);
+#define SCAN(NR)                                                                              \
+    hipLaunchKernelGGL(delta_scan_kernel<NR>, grid, block, 0, s, (const float*)qn,            \
+                       (const float*)kn, (const float*)vv, (const float*)beta,                \
+                       (const float*)decay, (float*)state, (const int*)cu_q,                  \
+                       (const int*)positions, (const int*)slots, (float*)o, H, G, D, E)
+    if (D <= 32) SCAN(8);
+    else if (D <= 64) SCAN(16);
+    else if (D <= 128) SCAN(32);
+    else if (D <= 256) SCAN(64);
+    else SCAN(128);
+#undef SCAN
+    return HYB_LAUNCH_OK();
+}
+
+}  // extern "C"

@@ -1291,7 +1291,8 @@ class ModelRunner:
             self._dec_dev.copy_(self._dec_host, non_blocking=True)
             if bucket is not None:
                 self.graphs[bucket].replay()
-                tokens = self._graph_out[bucket][:B]
+                tokens = self._graph_out[bucket]
+                tokens = tokens[:B] if tokens is not None else None
                 logits = self._graph_logits.get(bucket)
             else:
                 t = self._decode_tensors(B)
@@ -1331,7 +1332,7 @@ class ModelRunner:
 
     def _forward_and_sample(self, t: dict, score_only: bool = False) -> Optional[torch.Tensor]:
         hidden = self.model(t["input_ids"], t["positions"])
-        if score_only:
+        if score_only or self.cfg.score_only:
             # a scoring step: the logits of the asked rows are the result, nothing is drawn
             self._last_logits = self.model.lm_head.local_logits(hidden)
             return None
@@ -1346,9 +1347,14 @@ class ModelRunner:
             if logits.dtype != torch.float32:
                 from minivllm_amd.ops import hip
             if logits.dtype == torch.float32:
-                # the sampling kernel takes 16-bit logits; a 32-bit engine draws with the
-                # PyTorch sampler
-                return self.sampler(logits[..., :head.num_embeddings], temperatures).to(torch.int32)
+                # the sampling kernel takes 16-bit logits; a 32-bit engine draws with PyTorch
+                # ops (Gumbel arg-max, no host synchronisation: the step may be being captured)
+                lf = logits[..., :head.num_embeddings]
+                t = temperatures.float()
+                safe_t = torch.where(t > 0, t, torch.ones_like(t))
+                u = torch.rand_like(lf).clamp_(1e-20, 1.0 - 1e-7)
+                drawn = (lf / safe_t[:, None] - torch.log(-torch.log(u))).argmax(-1)
+                return torch.where(t > 0, drawn, lf.argmax(-1)).to(torch.int32)
             vals, idx = hip.sample_local(logits, temperatures, self.cfg.seed, step,
                                          vocab_offset=head.vocab_start,
                                          valid_vocab=head.num_embeddings)

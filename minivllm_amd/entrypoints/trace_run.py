@@ -69,7 +69,7 @@ def main(argv=None) -> int:
                          max_num_sequences=a.max_seqs, max_model_length=length,
                          max_num_batched_tokens=max(length, bs), eos=-1, enforce_eager=a.eager,
                          graph_batch_sizes=sorted({1, 2, a.max_seqs}), tuned_gemms=dense,
-                         tune_decode_gemms=dense, tune_prefill_gemms=dense))
+                         tune_decode_gemms=dense, tune_prefill_gemms=dense, score_only=True))
     os.makedirs(a.out, exist_ok=True)
     try:
         for line in sys.stdin:

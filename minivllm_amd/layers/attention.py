@@ -188,6 +188,11 @@ class SinkAttention(nn.Module):
         if not ctx.is_prefill:
             ops.sink_attention_decode(q, *a, ctx.block_tables, ctx.context_lens, self.scale,
                                       self.sink, gate, out)
+        elif q.is_cuda:
+            # one launch for every row of the step, decode riders included: a row's context is
+            # its position + 1 keys of its sequence
+            ops.sink_attention_step(q, *a, ctx.block_tables, ctx.row_seq, ctx.positions,
+                                    self.scale, self.sink, gate, out)
         else:
             Bd = ctx.num_decode_seqs
             if ctx.num_seqs > Bd:

@@ -267,6 +267,13 @@ def sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables, scale,
                                              scale, sink, gate, out)
 
 
+def sink_attention_step(q, k_cache, v_cache, block_tables, row_seq, positions, scale, sink, gate,
+                        out):
+    """GPU only: all rows of a prefill-form step in one launch (``hip_hybrid``)."""
+    return _hybrid().sink_attention_step(q, k_cache, v_cache, block_tables, row_seq, positions,
+                                         scale, sink, gate, out)
+
+
 def sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens, scale, sink, gate, out):
     return _seqmix(q).sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens,
                                             scale, sink, gate, out)

@@ -19,6 +19,12 @@ from .partials import ResidualSum, SplitKPartials      # the types live where CP
 _LIB_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
                          "_hip_kernels.so")
 _LIB_PATH = os.environ.get("MINIVLLM_HIP_LIB", _LIB_PATH)        # kernel experiments: another build
+if not os.path.exists(_LIB_PATH) and "MINIVLLM_HIP_LIB" not in os.environ:
+    try:                                   # a fresh checkout: build on first use
+        from minivllm_amd import build as _build
+        _build.build_hip(verbose=False)
+    except Exception:                      # noqa: BLE001  (no hipcc: the message below)
+        pass
 if not os.path.exists(_LIB_PATH):
     raise ImportError(
         f"{_LIB_PATH} is missing: build the HIP kernels first with "
