@@ -59,9 +59,10 @@ PHASE_PORT_OFFSET = {"dp": 101, "tp": 202, "tpc": 303, "l32k": 404}
 LONG_CONTEXT = dict(model="qwen3-32b", seq_len=32768, prefill_tokens=32768, batch=8)
 
 
-def make_config(args, model_name: str, world: int) -> EngineConfig:
-    model = model_preset(model_name)
-    if args.layers:
+def make_config(args, model_name, world: int) -> EngineConfig:
+    """``model_name``: a preset name, or a model configuration object of any family."""
+    model = model_preset(model_name) if isinstance(model_name, str) else model_name
+    if args.layers and isinstance(model_name, str):
         model.num_layers = args.layers          # debugging only; reported in the JSON
     port = int(os.environ.get("MASTER_PORT", args.port))
     return EngineConfig(
@@ -267,6 +268,70 @@ def bench_model(args, model_name: str, rank: int, world: int, replicas: bool = F
             eng.step()
     eng.exit()
     return res
+
+
+# ---------------------------------------------------------------- hybrid family, side by side
+HYBRID_SIZES = {
+    # name: (width, layers, query heads, kv heads, head size, dense intermediate size)
+    "w1024": (1024, 8, 16, 8, 128, 3072),
+    "w2048": (2048, 8, 16, 8, 128, 6144),
+}
+
+
+def hybrid_models(size: str, vocab: int = 32768, experts: int = 4, top: int = 2):
+    """(Natilix configuration, dense Qwen3-style configuration) of equal width, depth, head
+    geometry and active feed-forward parameters per token (top * 2 * ff = 3 * intermediate):
+    half of the hybrid's layers are attention, half delta rule, every layer has routed experts."""
+    from minivllm_amd.config import ModelConfig
+    from minivllm_amd.models.natilix import NatilixConfig
+    W, L, H, G, D, inter = HYBRID_SIZES[size]
+    ff = 3 * inter // (2 * top) // 64 * 64
+    rot = {"base": 10000.0, "dims": D, "scaling": None}
+    mlp = {"kind": "moe", "expert": {"ff": ff},
+           "router": {"experts": experts, "top": top, "groups": {"count": 2, "keep": 1}}}
+    layers = []
+    for i in range(L):
+        if i % 2 == 0:
+            layers.append({"type": "attention", "mlp": mlp,
+                           "mixer": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "rot": rot,
+                                     "scale": D ** -0.5, "v_mix": True}})
+        else:
+            layers.append({"type": "delta", "mlp": mlp,
+                           "mixer": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "conv": 4}})
+    hybrid = NatilixConfig.from_dict({"architecture": "Natilix", "vocab": vocab, "width": W,
+                                      "norm": {"eps": 1e-6}, "layers": layers,
+                                      "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31,
+                                                               "mul_cur": 17}},
+                                      "max_position": 8192}, name=f"natilix-{size}")
+    dense = ModelConfig(vocab_size=vocab, hidden_size=W, num_heads=H, num_kv_heads=G, head_dim=D,
+                        intermediate_size=inter, num_layers=L, max_position=8192,
+                        tie_word_embeddings=False, name=f"dense-{size}")
+    return hybrid, dense
+
+
+def hybrid_comparison(args) -> dict:
+    """Prefill and decode throughput of the hybrid family next to the dense decoder of the same
+    size, one GPU, same engine path as the headline measurement (``bench_model``)."""
+    out = {"metric": "prefill / decode tok/s, hybrid (attention + delta rule + routed experts) "
+                     "next to the dense decoder of equal size",
+           "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "dtype": "bf16", "data": "synthetic random token prompts, random-init weights",
+           "config": {"seq_len": args.seq_len, "decode_batch": args.batch,
+                      "prefill_tokens_per_step": args.prefill_tokens, "kv_block_size": args.block_size},
+           "sizes": {}}
+    for size in args.hybrid.split(","):
+        hybrid, dense = hybrid_models(size)
+        row = {}
+        for name, model in (("hybrid", hybrid), ("dense", dense)):
+            r = bench_model(args, model, 0, 1)
+            row[name] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in r.items()
+                         if k in ("prefill_tok_s", "prefill_ms_per_step", "decode_tok_s",
+                                  "decode_ms_per_step", "hipgraph_captured", "init_s")}
+        for k in ("prefill_tok_s", "decode_tok_s"):
+            if k in row["hybrid"] and k in row["dense"]:
+                row[f"hybrid_over_dense_{k}"] = round(row["hybrid"][k] / row["dense"][k], 3)
+        out["sizes"][size] = row
+    return out
 
 
 def _round(d):
@@ -568,8 +633,17 @@ def main():
                          "launch floor of a real N-GPU run; NOT a scaling number)")
     ap.add_argument("--p2p", action="store_true",
                     help="with --tp-shard: all-reduces by the peer-to-peer kernels in loop-back form")
+    ap.add_argument("--hybrid", default="",
+                    help="instead of the headline workload: the hybrid family (Natilix) next to "
+                         "the dense decoder of equal size; comma-separated sizes of "
+                         f"{sorted(HYBRID_SIZES)} (one GPU; --batch / --seq-len / --prefill-tokens "
+                         "/ --steps apply)")
     args = ap.parse_args()
 
+    if args.hybrid:
+        claim_stdout()
+        emit(hybrid_comparison(args))
+        return
     if os.environ.get("MINIVLLM_HANG_DUMP"):     # debugging aid: dump all stacks if stuck
         import faulthandler
         faulthandler.dump_traceback_later(int(os.environ["MINIVLLM_HANG_DUMP"]), repeat=False)

@@ -10,7 +10,7 @@
 
 using namespace hyb;
 
-constexpr int MAX_TAPS = 8;
+constexpr int MAX_TAPS = 32;
 
 // One workgroup per token row.  proj row = [q (G*D) | k (G*D) | v (H*E) | gate | b (H) | a (H)];
 // the three convolved blocks are contiguous at the row's start (C = 2GD + HE channels).

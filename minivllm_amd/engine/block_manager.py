@@ -351,6 +351,21 @@ class NativeBlockManager:
             bt.append(added)
         assert len(bt) == seq.num_blocks
 
+    def can_grow(self, seq: Sequence) -> bool:
+        return self.num_free_blocks >= seq.num_blocks - len(seq.block_table)
+
+    def grow(self, seq: Sequence) -> None:
+        """See :meth:`BlockManager.grow` (one library call per missing block, each asking for
+        the block that the first token beyond the table starts; nothing is published)."""
+        bt = seq.block_table
+        while len(bt) < seq.num_blocks:
+            added = self._lib.mvl_bm_append(self._h, len(bt), bt[-1] if bt else -1,
+                                            bt[-2] if len(bt) > 1 else -1,
+                                            len(bt) * self.block_size + 1, None)
+            if added < 0:
+                raise RuntimeError("grow() without a free block (check can_grow first)")
+            bt.append(added)
+
     def append_ahead(self, seq: Sequence) -> None:
         """See :meth:`BlockManager.append_ahead`."""
         bt = seq.block_table

@@ -177,7 +177,7 @@ class ModelRunner:
         # models that bring their own cache layout (attention layers with their own head sizes,
         # layers with per-sequence recurrent state): see ``allocate_kv_cache``
         self.hybrid = hasattr(self.model, "state_layers")
-        self.needs_aux_rows = hasattr(self.model, "aux_embedding_rows")
+        self.needs_aux_rows = bool(getattr(self.model, "needs_aux_rows", False))
         self.num_state_slots = cfg.max_num_sequences if self.hybrid and self.model.state_layers() else 0
         fold = cfg.fold_norm_weights
         if fold is None:
@@ -1052,7 +1052,7 @@ class ModelRunner:
         set_context(False, slot_mapping=t["slot_mapping"], context_lens=t["context_lens"],
                     block_tables=t["block_tables"], positions=t["positions"],
                     max_context_len=b.max_context_len, num_seqs=B, positions_in_context=True,
-                    state_slots=t["state_slots"], aux_rows=t["aux_rows"])
+                    state_slots=t.get("state_slots"), aux_rows=t.get("aux_rows"))
         tokens = self._forward_and_sample(t)
         reset_context()
         return tokens
@@ -1245,15 +1245,18 @@ class ModelRunner:
     def _decode_tensors(self, n: int):
         d = self._dec_dev
         MB = self.max_blocks_per_seq
-        return dict(input_ids=self._dec_view(d, "input_ids", n),
-                    positions=self._dec_view(d, "positions", n),
-                    slot_mapping=self._dec_view(d, "slot_mapping", n),
-                    context_lens=self._dec_view(d, "context_lens", n),
-                    temperatures=self._dec_view(d, "temperatures", n).view(torch.float32),
-                    step=self._dec_view(d, "misc"),
-                    aux_rows=self._dec_view(d, "aux_rows", n) if self.needs_aux_rows else None,
-                    state_slots=self._dec_view(d, "state_slots", n) if self.num_state_slots else None,
-                    block_tables=self._dec_view(d, "block_tables", n * MB).view(n, MB))
+        t = dict(input_ids=self._dec_view(d, "input_ids", n),
+                 positions=self._dec_view(d, "positions", n),
+                 slot_mapping=self._dec_view(d, "slot_mapping", n),
+                 context_lens=self._dec_view(d, "context_lens", n),
+                 temperatures=self._dec_view(d, "temperatures", n).view(torch.float32),
+                 step=self._dec_view(d, "misc"),
+                 block_tables=self._dec_view(d, "block_tables", n * MB).view(n, MB))
+        if self.needs_aux_rows:
+            t["aux_rows"] = self._dec_view(d, "aux_rows", n)
+        if self.num_state_slots:
+            t["state_slots"] = self._dec_view(d, "state_slots", n)
+        return t
 
     # -------------------------------------------------------------- execute
     def _enqueue_prefill(self, b: Batch, pg_key, warmup: bool = False):
@@ -1271,9 +1274,9 @@ class ModelRunner:
                     context_lens=t["context_lens"] if b.num_decode_seqs else None,
                     max_context_len=b.max_context_len, total_k_tokens=b.num_prefill_k_tokens,
                     prefill_items=None if warmup else t["prefill_items"],
-                    positions_in_context=True, state_slots=t["state_slots"],
-                    aux_rows=t["aux_rows"], row_seq=t["row_seq"], logit_rows=t["logit_rows"])
-        tokens = self._forward_and_sample(t, score_only=t["logit_rows"] is not None)
+                    positions_in_context=True, state_slots=t.get("state_slots"),
+                    aux_rows=t.get("aux_rows"), row_seq=t.get("row_seq"), logit_rows=t.get("logit_rows"))
+        tokens = self._forward_and_sample(t, score_only=t.get("logit_rows") is not None)
         return tokens, self._last_logits
 
     def execute(self, b: Batch, warmup: bool = False, pg_key=_PG_KEY_UNSET) -> Optional[List[int]]:
@@ -1299,8 +1302,8 @@ class ModelRunner:
                 set_context(False, slot_mapping=t["slot_mapping"], context_lens=t["context_lens"],
                             block_tables=t["block_tables"], positions=t["positions"],
                             max_context_len=b.max_context_len, num_seqs=B,
-                            positions_in_context=True, state_slots=t["state_slots"],
-                            aux_rows=t["aux_rows"])
+                            positions_in_context=True, state_slots=t.get("state_slots"),
+                            aux_rows=t.get("aux_rows"))
                 tokens = self._forward_and_sample(t)
                 logits = self._last_logits
         reset_context()
@@ -1487,8 +1490,8 @@ class ModelRunner:
                 set_context(False, slot_mapping=t["slot_mapping"], context_lens=t["context_lens"],
                             block_tables=t["block_tables"], positions=t["positions"],
                             max_context_len=self.cfg.max_model_length, num_seqs=bs,
-                            positions_in_context=True, state_slots=t["state_slots"],
-                            aux_rows=t["aux_rows"])
+                            positions_in_context=True, state_slots=t.get("state_slots"),
+                            aux_rows=t.get("aux_rows"))
                 out = self._forward_and_sample(t)
                 reset_context()
                 return out

@@ -29,9 +29,9 @@ class GatedDeltaRule(nn.Module):
         self.num_heads, self.num_kv_heads, self.head_dim, self.v_head_dim = H, G, D, E
         self.taps, self.eps = conv_taps, eps
         f32 = dict(dtype=torch.float32)
-        self.conv_q = nn.Parameter(torch.zeros(G * D, conv_taps, **f32), requires_grad=False)
-        self.conv_k = nn.Parameter(torch.zeros(G * D, conv_taps, **f32), requires_grad=False)
-        self.conv_v = nn.Parameter(torch.zeros(H * E, conv_taps, **f32), requires_grad=False)
+        # taps of the q, k and v channels stacked in that order (last column = current token)
+        self.conv_weight = nn.Parameter(torch.zeros(2 * G * D + H * E, conv_taps, **f32),
+                                        requires_grad=False)
         self.A_log = nn.Parameter(torch.zeros(H, **f32), requires_grad=False)
         self.dt_bias = nn.Parameter(torch.zeros(H, **f32), requires_grad=False)
         self.norm_weight = nn.Parameter(torch.ones(E, **f32), requires_grad=False)
@@ -59,7 +59,7 @@ class GatedDeltaRule(nn.Module):
         cu_q = ctx.cu_seqlens_q if ctx.is_prefill else None
         lay = (cu_q, ctx.positions, ctx.state_slots)
         qn, kn, vv, beta, decay = ops.delta_prepare(
-            q.view(T, G, D), k.view(T, G, D), v.view(T, H, E), b, a, self.conv_q, self.conv_k,
-            self.conv_v, self.A_log, self.dt_bias, self.conv_state, *lay, row_seq=ctx.row_seq)
+            q.view(T, G, D), k.view(T, G, D), v.view(T, H, E), b, a, self.conv_weight,
+            self.A_log, self.dt_bias, self.conv_state, *lay, row_seq=ctx.row_seq)
         o = ops.delta_scan(qn, kn, vv, beta, decay, self.state, *lay)
         return ops.gated_head_norm(o, self.norm_weight, gate, self.eps, out_dtype).view(T, H * E)

@@ -278,9 +278,13 @@ class NatilixForCausalLM(nn.Module):
     def state_layers(self):
         return [l.mix.core for l in self.model.layers if l.kind == "delta"]
 
+    @property
+    def needs_aux_rows(self) -> bool:
+        """The batch must carry a row of the second embedding table for every token."""
+        return self.model.bigram is not None
+
     def aux_embedding_rows(self, tokens, prev_tokens):
-        b = self.model.bigram
-        return None if b is None else b.rows_for(tokens, prev_tokens)
+        return self.model.bigram.rows_for(tokens, prev_tokens)
 
     # ---- weights -----------------------------------------------------------------------
     @torch.no_grad()
@@ -328,8 +332,10 @@ class NatilixForCausalLM(nn.Module):
             core, order = mix.core, ["q", "k", "v", "g", "b", "a"]
             if key in order:
                 return _put_rows(mix.in_proj, core.split_sizes(), order.index(key), t)
-            simple = {"q.conv": core.conv_q, "k.conv": core.conv_k, "v.conv": core.conv_v,
-                      "A_log": core.A_log, "dt_bias": core.dt_bias, "norm": core.norm_weight}
+            convs = ["q.conv", "k.conv", "v.conv"]
+            if key in convs:
+                return _put_rows(core.conv_weight, core.split_sizes()[:3], convs.index(key), t)
+            simple = {"A_log": core.A_log, "dt_bias": core.dt_bias, "norm": core.norm_weight}
             if key in simple:
                 return _put(simple[key], t)
         raise KeyError(f"checkpoint tensor {name!r} has no parameter")

@@ -279,14 +279,14 @@ def sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens, scale
                                             scale, sink, gate, out)
 
 
-def delta_prepare(q, k, v, b, a, wq, wk, wv, a_log, dt_bias, conv_state, cu_q, positions, slots,
+def delta_prepare(q, k, v, b, a, conv_w, a_log, dt_bias, conv_state, cu_q, positions, slots,
                   row_seq=None):
     """``row_seq`` [T] (GPU, prefill-form steps): the sequence of each row, -1 for rows that
     belong to none; the CPU form walks ``cu_q`` instead."""
     if _on_gpu(q):
-        return _hybrid().delta_prepare(q, k, v, b, a, wq, wk, wv, a_log, dt_bias, conv_state,
+        return _hybrid().delta_prepare(q, k, v, b, a, conv_w, a_log, dt_bias, conv_state,
                                        cu_q, positions, slots, row_seq)
-    return torch_seqmix.delta_prepare(q, k, v, b, a, wq, wk, wv, a_log, dt_bias, conv_state,
+    return torch_seqmix.delta_prepare(q, k, v, b, a, conv_w, a_log, dt_bias, conv_state,
                                       cu_q, positions, slots)
 
 

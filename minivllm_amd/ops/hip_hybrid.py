@@ -167,7 +167,7 @@ def sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens, scale
 
 
 # ------------------------------------------------------------------ gated delta rule
-def delta_prepare(q, k, v, b, a, wq, wk, wv, a_log, dt_bias, conv_state, cu_q, positions, slots,
+def delta_prepare(q, k, v, b, a, conv_w, a_log, dt_bias, conv_state, cu_q, positions, slots,
                   row_seq):
     T, G, D = q.shape
     H, E = v.shape[1], v.shape[2]
@@ -180,11 +180,8 @@ def delta_prepare(q, k, v, b, a, wq, wk, wv, a_log, dt_bias, conv_state, cu_q, p
                       and a.stride(0) == rs)
     b_off, a_off = (b.data_ptr() - base) // es, (a.data_ptr() - base) // es
     dev = q.device
-    conv_w = getattr(wq, "_stacked_conv", None)
-    if conv_w is None:                     # stacked once per layer, kept with the parameter
-        conv_w = torch.cat([wq, wk, wv], 0).float().contiguous()
-        wq._stacked_conv = conv_w
-    taps = conv_w.shape[1]
+    taps = _f32(conv_w).shape[1]
+    assert conv_w.shape[0] == 2 * G * D + H * E
     f = dict(dtype=torch.float32, device=dev)
     qn, kn = torch.empty((T, G, D), **f), torch.empty((T, G, D), **f)
     vv, beta, decay = torch.empty((T, H, E), **f), torch.empty((T, H), **f), torch.empty((T, H), **f)

@@ -153,7 +153,7 @@ def sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens, scale
 
 
 # ------------------------------------------------------------------ gated delta rule
-def delta_prepare(q, k, v, b, a, wq, wk, wv, a_log, dt_bias, conv_state, cu_q, positions, slots):
+def delta_prepare(q, k, v, b, a, conv_w, a_log, dt_bias, conv_state, cu_q, positions, slots):
     """Short causal convolution + silu on q / k / v (their last taps-1 inputs per sequence live
     in ``conv_state`` [slots, taps-1, Cq+Ck+Cv] fp32 and are replaced by this step's), unit
     vectors for q (times D^-1/2) and k, beta = sigmoid(b), decay = exp(-exp(A_log) softplus(a +
@@ -161,7 +161,7 @@ def delta_prepare(q, k, v, b, a, wq, wk, wv, a_log, dt_bias, conv_state, cu_q, p
     T, G, D = q.shape
     H, E = v.shape[1], v.shape[2]
     x = torch.cat([q.reshape(T, -1), k.reshape(T, -1), v.reshape(T, -1)], -1).float()
-    w = torch.cat([wq, wk, wv], 0).float()                             # [C, taps]
+    w = conv_w.float()                                                 # [C, taps]: q, k, v rows
     taps = w.shape[1]
     y = torch.empty_like(x)
     B = slots.shape[0]

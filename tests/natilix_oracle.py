@@ -145,9 +145,26 @@ def grouped_top_experts(z: torch.Tensor, top: int, groups: int, keep: int):
     return ids.tolist(), s[ids]
 
 
-def routed_ffn(h: torch.Tensor, router, ups, downs, top, groups, keep):
+def routing_margin(z: torch.Tensor, top: int, groups: int, keep: int) -> float:
+    """How far the routing decision for logits z is from flipping: the smallest gap between a
+    kept and a dropped group's best score, or between a chosen and an eligible unchosen score."""
+    s = torch.softmax(z, -1)
+    per = s.shape[0] // groups
+    best = s.view(groups, per).max(-1).values.sort(descending=True).values
+    m = float(best[keep - 1] - best[keep]) if keep < groups else 1.0
+    ids, _ = grouped_top_experts(z, top, groups, keep)
+    kept = torch.topk(s.view(groups, per).max(-1).values, keep).indices.tolist()
+    rest = [float(s[e]) for gi in kept for e in range(gi * per, (gi + 1) * per) if e not in ids]
+    if rest:
+        m = min(m, float(s[ids].min()) - max(rest))
+    return m
+
+
+def routed_ffn(h: torch.Tensor, router, ups, downs, top, groups, keep, margins=None):
     out = torch.zeros(h.shape[0], downs[0].shape[0], dtype=h.dtype)
     for t in range(h.shape[0]):
+        if margins is not None:
+            margins[t] = min(margins[t], routing_margin(router @ h[t], top, groups, keep))
         ids, w = grouped_top_experts(router @ h[t], top, groups, keep)
         for e, we in zip(ids, w):
             out[t] += we * (downs[e] @ gelu_erf(ups[e] @ h[t]))
@@ -217,12 +234,15 @@ class Oracle:
     def feed(self, tokens: List[int]) -> torch.Tensor:
         cfg, w, st = self.cfg, self.w, self.state
         T = len(tokens)
-        bg = cfg["embedding"]["bigram"]
-        rows = bigram_rows(tokens, st["prev"], bg["mul_prev"], bg["mul_cur"], bg["buckets"])
-        x = w["embed"][tokens] + w["bigram"][rows]
+        x = w["embed"][tokens]
+        bg = (cfg.get("embedding") or {}).get("bigram")
+        if bg:
+            rows = bigram_rows(tokens, st["prev"], bg["mul_prev"], bg["mul_cur"], bg["buckets"])
+            x = x + w["bigram"][rows]
         pos = torch.arange(st["n"], st["n"] + T)
         shared = {}
         self.trace = []
+        self.margin = [1.0] * T          # per token: the closest routing decision of any layer
         for i, layer in enumerate(cfg["layers"]):
             p, ls, m = f"l{i}.", st["layers"][i], layer["mixer"]
             h = norm_around_zero(x, w[p + "norm1"], self.eps)
@@ -235,7 +255,7 @@ class Oracle:
                 h = norm_around_zero(x, w[p + "norm2"], self.eps)
                 y = routed_ffn(h, w[p + "mlp.router"], [w[f"{p}mlp.e{e}.up"] for e in range(E)],
                                [w[f"{p}mlp.e{e}.down"] for e in range(E)], r["top"],
-                               r["groups"]["count"], r["groups"]["keep"])
+                               r["groups"]["count"], r["groups"]["keep"], margins=self.margin)
                 x = x + norm_around_zero(y, w[p + "norm2b"], self.eps)
             self.trace.append(x.clone())
         st["n"] += T

@@ -139,8 +139,7 @@ def test_delta_prepare_and_scan(dt, H, G, D, E, taps):
     torch.manual_seed(3)
     slots_n = 6
     sizes = [G * D, G * D, H * E, H * E, H, H]
-    wq, wk, wv = (0.5 * torch.randn(G * D, taps), 0.5 * torch.randn(G * D, taps),
-                  0.5 * torch.randn(H * E, taps))
+    conv_w = 0.5 * torch.randn(2 * G * D + H * E, taps)
     a_log, dt_bias = -1 + 0.5 * torch.randn(H), torch.randn(H)
     state0 = torch.randn(slots_n, H, D, E)
     conv0 = torch.randn(slots_n, max(taps - 1, 0), 2 * G * D + H * E)
@@ -169,7 +168,7 @@ def test_delta_prepare_and_scan(dt, H, G, D, E, taps):
                 sl = torch.cat([slots, torch.tensor([-1], dtype=torch.int32)])
             proj = to(torch.randn(T, sum(sizes)).to(dt))
             q, k, v, gate, b_, a_ = proj.split(sizes, -1)
-            args = (q.view(T, G, D), k.view(T, G, D), v.view(T, H, E), b_, a_, to(wq), to(wk), to(wv),
+            args = (q.view(T, G, D), k.view(T, G, D), v.view(T, H, E), b_, a_, to(conv_w),
                     to(a_log), to(dt_bias), conv, to(cu_q), to(pos), to(sl))
             prep = mod.delta_prepare(*args, to(row_seq)) if name == "gpu" else mod.delta_prepare(*args)
             o = mod.delta_scan(*prep, state, to(cu_q), to(pos), to(sl))
