@@ -41,14 +41,14 @@ sink_attention_rows_kernel(const T* __restrict__ q, long q_row, long q_head,
                            const int* __restrict__ row_seq, const int* __restrict__ lens,
                            int len_add, const float* __restrict__ sink,
                            const T* __restrict__ gate, long gate_row, T* __restrict__ out,
-                           float scale, int H, int G, int D, int E, int vec_ok) {
+                           float scale, int H, int G, int D, int E, int vec_ok, int seq_base) {
     extern __shared__ float sm[];
     const int R = H / G;
     const int chunks = (R + RC - 1) / RC;
     const long t = blockIdx.x;
     const int g = blockIdx.y / chunks, h0 = g * R + (blockIdx.y % chunks) * RC;
     const int nr = min(RC, g * R + R - h0);
-    const int b = row_seq ? row_seq[t] : (int)t;
+    const int b = row_seq ? row_seq[t] - seq_base : (int)t;      // seq_base: first table row
     if (b < 0) return;
     const int ctx = lens[row_seq ? t : b] + len_add;
     if (ctx <= 0) return;
@@ -168,7 +168,225 @@ sink_attention_rows_kernel(const T* __restrict__ q, long q_row, long q_head,
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// Prompt portions: tiles on the matrix cores, everything in fp32.
+//
+// Workgroup = 4 waves = 128 consecutive queries of one (sequence, query head); a wave owns 32 of
+// them.  Keys are walked in tiles of 32 through LDS (K tile [32][DP+1], V tile [32][EP], both
+// widened to fp32 on the way in).  Scores are computed transposed, S^T = K Q^T, with
+// v_mfma_f32_32x32x2_f32: a lane then holds 16 keys of ONE query (column lane%32), so the
+// running maximum and sum are per-lane values (one exchange with lane^32), and the
+// accumulator registers are, as they stand, the B operand of O^T += V^T P^T: register r of
+// both halves of the wave names key 8(r/4) + 4(lane/32) + r%4, which is the key row the A
+// operand (V^T) is read from.  The sink initialises the running maximum (sum 1).  DP / EP:
+// head sizes rounded up to the template's register arrays (padding columns of K are zeroed).
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+template <typename T, int DP, int EP>
+__global__ void __launch_bounds__(256)
+sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
+                            const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+                            const int* __restrict__ block_tables, int max_blocks, int block_size,
+                            const int* __restrict__ cu_q, const int* __restrict__ positions,
+                            const float* __restrict__ sink, const T* __restrict__ gate,
+                            long gate_row, T* __restrict__ out, float scale, int H, int G, int D,
+                            int E, int seq0, int vec_k, int vec_v) {
+    extern __shared__ float sm[];
+    constexpr int KS = DP + 1;
+    float* Ks = sm;
+    float* Vs = sm + 32 * KS;
+    const int b = blockIdx.x + seq0, tile = blockIdx.y, h = blockIdx.z;
+    const int row0 = cu_q[b], qlen = cu_q[b + 1] - row0;
+    if (tile * 128 >= qlen) return;
+    const int start = positions[row0];
+    const int g = h / (H / G);
+    const int* table = block_tables + (long)b * max_blocks;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, half = lane >> 5, l32 = lane & 31;
+    const int qi = tile * 128 + wave * 32 + l32;
+    const bool qok = qi < qlen;
+    const int qpos = start + qi;
+
+    float qreg[DP / 2];
+    {
+        const T* qp = q + (long)(row0 + (qok ? qi : 0)) * q_row + (long)h * q_head;
+#pragma unroll
+        for (int s = 0; s < DP / 2; ++s) {
+            const int d = 2 * s + half;
+            qreg[s] = (qok && d < D) ? ld(qp + d) * scale : 0.f;
+        }
+    }
+    for (int i = tid; i < 32 * (KS - D); i += 256) {          // padding columns of K stay zero
+        const int key = i / (KS - D), c = D + i - key * (KS - D);
+        Ks[key * KS + c] = 0.f;
+    }
+    float m = sink[h], lsum = 1.f;
+    f32x16 oacc[EP / 32];
+#pragma unroll
+    for (int eb = 0; eb < EP / 32; ++eb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[eb][r] = 0.f;
+
+    const int wg_ctx = start + min(qlen, tile * 128 + 128);            // keys this workgroup needs
+    const bool wave_live = tile * 128 + wave * 32 < qlen;
+    const int wave_last = start + min(qlen - 1, tile * 128 + wave * 32 + 31);
+
+    for (int k0 = 0; k0 < wg_ctx; k0 += 32) {
+        // ---- K and V tile into LDS
+        if (vec_k) {
+            const int D4 = D >> 2;
+            for (int i = tid; i < 32 * D4; i += 256) {
+                const int key = i / D4, c = (i - key * D4) << 2, j = k0 + key;
+                float v4[4] = {0.f, 0.f, 0.f, 0.f};
+                if (j < wg_ctx) {
+                    const long slot = (long)table[j / block_size] * block_size + j % block_size;
+                    Vec4<T>::load(k_cache + (slot * G + g) * (long)D + c, v4);
+                }
+                float* dst = Ks + key * KS + c;
+                dst[0] = v4[0]; dst[1] = v4[1]; dst[2] = v4[2]; dst[3] = v4[3];
+            }
+        } else {
+            for (int i = tid; i < 32 * D; i += 256) {
+                const int key = i / D, c = i - key * D, j = k0 + key;
+                float v = 0.f;
+                if (j < wg_ctx) {
+                    const long slot = (long)table[j / block_size] * block_size + j % block_size;
+                    v = ld(k_cache + (slot * G + g) * (long)D + c);
+                }
+                Ks[key * KS + c] = v;
+            }
+        }
+        if (vec_v) {
+            const int E4 = E >> 2;
+            for (int i = tid; i < 32 * E4; i += 256) {
+                const int key = i / E4, c = (i - key * E4) << 2, j = k0 + key;
+                float v4[4] = {0.f, 0.f, 0.f, 0.f};
+                if (j < wg_ctx) {
+                    const long slot = (long)table[j / block_size] * block_size + j % block_size;
+                    Vec4<T>::load(v_cache + (slot * G + g) * (long)E + c, v4);
+                }
+                float* dst = Vs + key * EP + c;
+                dst[0] = v4[0]; dst[1] = v4[1]; dst[2] = v4[2]; dst[3] = v4[3];
+            }
+        } else {
+            for (int i = tid; i < 32 * E; i += 256) {
+                const int key = i / E, c = i - key * E, j = k0 + key;
+                float v = 0.f;
+                if (j < wg_ctx) {
+                    const long slot = (long)table[j / block_size] * block_size + j % block_size;
+                    v = ld(v_cache + (slot * G + g) * (long)E + c);
+                }
+                Vs[key * EP + c] = v;
+            }
+        }
+        __syncthreads();
+        if (wave_live && k0 <= wave_last) {
+            f32x16 sacc;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+            const float* ka = Ks + l32 * KS + half;
+#pragma unroll
+            for (int s = 0; s < DP / 2; ++s)
+                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[2 * s], qreg[s], sacc, 0, 0, 0);
+            float mt = -INFINITY;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int key = k0 + 8 * (r >> 2) + 4 * half + (r & 3);
+                const float v = (qok && key <= qpos) ? sacc[r] : -INFINITY;
+                sacc[r] = v;
+                mt = fmaxf(mt, v);
+            }
+            mt = fmaxf(mt, __shfl_xor(mt, 32, kWave));
+            const float mnew = fmaxf(m, mt);
+            const float alpha = expf(m - mnew);
+            float ps = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float p = expf(sacc[r] - mnew);
+                sacc[r] = p;
+                ps += p;
+            }
+            ps += __shfl_xor(ps, 32, kWave);
+            lsum = lsum * alpha + ps;
+            m = mnew;
+#pragma unroll
+            for (int eb = 0; eb < EP / 32; ++eb) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) oacc[eb][r] *= alpha;
+                const float* va = Vs + (4 * half) * EP + eb * 32 + l32;
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    oacc[eb] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+                        va[(8 * (r >> 2) + (r & 3)) * EP], sacc[r], oacc[eb], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+    if (!qok) return;
+    const long row = row0 + qi;
+    float f = 1.f / lsum;
+    if (gate) f *= sigmoidf_(ld(gate + row * gate_row + h));
+    T* op = out + (row * H + h) * (long)E;
+#pragma unroll
+    for (int eb = 0; eb < EP / 32; ++eb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int e = eb * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+            if (e < E) st(op + e, oacc[eb][r] * f);
+        }
+}
+
+template <typename T, int DP, int EP>
+static int launch_tiles(const void* q, long q_row, long q_head, const void* k_cache,
+                        const void* v_cache, const void* block_tables, int max_blocks,
+                        int block_size, const void* cu_q, const void* positions, const void* sink,
+                        const void* gate, long gate_row, void* out, float scale, int nseq,
+                        int seq0, int max_q, int H, int G, int D, int E, int esize,
+                        hipStream_t s) {
+    const size_t lds = (32 * (DP + 1) + 32 * EP) * sizeof(float);
+    const int vec_k = (D % 4 == 0) && ((size_t)k_cache % 16 == 0);
+    const int vec_v = (E % 4 == 0) && ((size_t)v_cache % 16 == 0);
+    hipLaunchKernelGGL((sink_attention_tiles_kernel<T, DP, EP>), dim3(nseq, (max_q + 127) / 128, H),
+                       dim3(256), lds, s, (const T*)q, q_row, q_head, (const T*)k_cache,
+                       (const T*)v_cache, (const int*)block_tables, max_blocks, block_size,
+                       (const int*)cu_q, (const int*)positions, (const float*)sink,
+                       (const T*)gate, gate_row, (T*)out, scale, H, G, D, E, seq0, vec_k, vec_v);
+    return HYB_LAUNCH_OK();
+}
+
 extern "C" {
+
+// 1 when the tile kernel has an instance for these head sizes (else the row kernel serves)
+int hyb_sink_attention_tiles_ok(int D, int E) { return D <= 256 && E <= 256 && !(D > 128 && E > 128); }
+
+// Sequences seq0 .. seq0 + nseq - 1 of a prefill-form step (cu_q / block_tables indexed by the
+// absolute sequence number); max_q: longest portion among them.
+int hyb_sink_attention_tiles(const void* q, long q_row, long q_head, const void* k_cache,
+                             const void* v_cache, const void* block_tables, int max_blocks,
+                             int block_size, const void* cu_q, const void* positions,
+                             const void* sink, const void* gate, long gate_row, void* out,
+                             float scale, int nseq, int seq0, int max_q, int H, int G, int D,
+                             int E, int dt, hipStream_t s) {
+    if (nseq <= 0 || max_q <= 0) return 0;
+    if (G <= 0 || H % G || !hyb_sink_attention_tiles_ok(D, E)) return 1;
+#define TILES_ARGS q, q_row, q_head, k_cache, v_cache, block_tables, max_blocks, block_size, cu_q, \
+                   positions, sink, gate, gate_row, out, scale, nseq, seq0, max_q, H, G, D, E
+#define TILES_E(T, DP, esz)                                                   \
+    do {                                                                      \
+        if (E <= 64) return launch_tiles<T, DP, 64>(TILES_ARGS, esz, s);      \
+        if (E <= 128) return launch_tiles<T, DP, 128>(TILES_ARGS, esz, s);    \
+        if (DP <= 128) return launch_tiles<T, (DP <= 128 ? DP : 64), 256>(TILES_ARGS, esz, s); \
+        return 1;                                                             \
+    } while (0)
+#define TILES_D(T, esz)                                   \
+    do {                                                  \
+        if (D <= 64) TILES_E(T, 64, esz);                 \
+        else if (D <= 128) TILES_E(T, 128, esz);          \
+        else TILES_E(T, 256, esz);                        \
+    } while (0)
+    if (dt == 0) TILES_D(hyb::bf16_t, 2);
+    else if (dt == 2) TILES_D(float, 4);
+    return 1;
+}
 
 // q: [rows, H, D] with strides (q_row, q_head, 1); caches contiguous [blocks, block, G, D|E];
 // out contiguous [rows, H, E]; gate [rows, H] with row stride gate_row (or null).
@@ -176,8 +394,8 @@ int hyb_sink_attention_rows(const void* q, long q_row, long q_head, const void* 
                             const void* v_cache, const void* block_tables, int max_blocks,
                             int block_size, const void* row_seq, const void* lens, int len_add,
                             const void* sink, const void* gate, long gate_row, void* out,
-                            float scale, long rows, int H, int G, int D, int E, int dt,
-                            hipStream_t s) {
+                            float scale, long rows, int H, int G, int D, int E, int seq_base,
+                            int dt, hipStream_t s) {
     if (rows <= 0) return 0;
     if (G <= 0 || H % G || RC * E > NACC * TILE || D > 1024) return 1;
     const int R = H / G, chunks = (R + RC - 1) / RC;
@@ -190,7 +408,7 @@ int hyb_sink_attention_rows(const void* q, long q_row, long q_head, const void* 
                                         (const int*)block_tables, max_blocks, block_size,
                                         (const int*)row_seq, (const int*)lens, len_add,
                                         (const float*)sink, (const T*)gate, gate_row, (T*)out,
-                                        scale, H, G, D, E, vec_ok));
+                                        scale, H, G, D, E, vec_ok, seq_base));
     return HYB_LAUNCH_OK();
 }
 

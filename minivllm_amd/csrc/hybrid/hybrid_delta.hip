@@ -104,8 +104,14 @@ __global__ void delta_conv_tail_kernel(const T* __restrict__ proj, long row_stri
 // The recurrence.  A state column S[:, e] evolves independently of the others:
 //   u_e = beta (v_e - g sum_d S[d,e] k_d);  S[d,e] <- g S[d,e] + k_d u_e;  o_e = sum_d S[d,e] q_d
 // so a column is owned by 4 neighbouring lanes, lane r holding d in [r*NR, (r+1)*NR) in
-// registers (D <= 4*NR, missing d padded with zeros).  Workgroup = 64 columns of one (sequence,
-// head); tokens are walked in order with the next token's k / q loads issued ahead.
+// registers (D <= 4*NR, missing d padded with zeros); the two sums over d close with two
+// exchanges inside the quad.  Workgroup = 64 columns of one (sequence, head).  The tokens'
+// operands (k, q of the head: shared by all columns; v of the 64 columns; beta, decay) are
+// staged through LDS in chunks of CT tokens, double-buffered: the next chunk's global loads are
+// in flight while the current chunk's steps run, and a step reads its k / q slice with 16-byte
+// LDS reads (per-lane global loads of these shared vectors were what bound the first version).
+template <int NR> struct ScanChunk { static constexpr int tokens = NR >= 64 ? 8 : 16; };
+
 template <int NR>
 __global__ void __launch_bounds__(256)
 delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
@@ -113,66 +119,125 @@ delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
                   const float* __restrict__ decay, float* __restrict__ state,
                   const int* __restrict__ cu_q, const int* __restrict__ positions,
                   const int* __restrict__ slots, float* __restrict__ o, int H, int G, int D, int E) {
+    constexpr int CT = ScanChunk<NR>::tokens;
+    constexpr int RS = NR + 4;                 // padded slice: the 4 lanes of a quad hit 4 bank groups
+    constexpr int KQ = CT * 4 * RS;            // floats of one k (or q) chunk image
+    constexpr int BUF = 2 * KQ + CT * 64 + 2 * CT;
+    constexpr int NLD = (2 * CT * 4 * NR + CT * 64 + 2 * CT + 255) / 256;   // staged floats per thread
+    extern __shared__ float sm[];
     const int b = blockIdx.x, h = blockIdx.y;
     const int slot = slots[b];
     if (slot < 0) return;
     const long first = cu_q ? cu_q[b] : b;
     const int n = cu_q ? cu_q[b + 1] - cu_q[b] : 1;
     if (n <= 0) return;
-    const int r = threadIdx.x & 3;
-    const int e = blockIdx.z * 64 + (threadIdx.x >> 2);
+    const int tid = threadIdx.x, r = tid & 3, c = tid >> 2;
+    const int e0 = blockIdx.z * 64, e = e0 + c;
     const bool col = e < E;
     const int g = h / (H / G);
     const int d0 = r * NR;
     float S[NR];
-    float* sp = state + (((long)slot * H + h) * D) * E + e;
+    float* sp = state + (((long)slot * H + h) * D) * E + (col ? e : 0);
     const bool has_past = positions[first] > 0;
 #pragma unroll
     for (int i = 0; i < NR; ++i)
         S[i] = (has_past && col && d0 + i < D) ? sp[(long)(d0 + i) * E] : 0.f;
-    float kc[NR], qc[NR];
-    auto load_kq = [&](long t, float* kk, float* qq) {
-        const float* kp = kn + (t * G + g) * (long)D + d0;
-        const float* qp = qn + (t * G + g) * (long)D + d0;
+
+    // staging: item j of a chunk = one float of k, q (padded to 4*NR per token), v, beta, decay
+    auto fetch = [&](int chunk, float* reg) {
+        const long t0 = first + (long)chunk * CT;
+        const int nt = min(CT, n - chunk * CT);
 #pragma unroll
-        for (int i = 0; i < NR; ++i) {
-            const bool ok = d0 + i < D;
-            kk[i] = ok ? kp[i] : 0.f;
-            qq[i] = ok ? qp[i] : 0.f;
+        for (int x = 0; x < NLD; ++x) {
+            const int j = tid + x * 256;
+            float v = 0.f;
+            if (j < 2 * CT * 4 * NR) {
+                const int which = j / (CT * 4 * NR), jj = j - which * (CT * 4 * NR);
+                const int tok = jj / (4 * NR), d = jj - tok * (4 * NR);
+                if (tok < nt && d < D)
+                    v = (which ? qn : kn)[((t0 + tok) * G + g) * (long)D + d];
+            } else if (j < 2 * CT * 4 * NR + CT * 64) {
+                const int jj = j - 2 * CT * 4 * NR, tok = jj >> 6, cc = jj & 63;
+                if (tok < nt && e0 + cc < E) v = vv[((t0 + tok) * H + h) * (long)E + e0 + cc];
+            } else if (j < 2 * CT * 4 * NR + CT * 64 + 2 * CT) {
+                const int jj = j - 2 * CT * 4 * NR - CT * 64, tok = jj % CT;
+                if (tok < nt) v = (jj < CT ? beta : decay)[(t0 + tok) * H + h];
+            }
+            reg[x] = v;
         }
     };
-    load_kq(first, kc, qc);
-    for (int s = 0; s < n; ++s) {
-        const long t = first + s;
-        float kx[NR], qx[NR];
-        if (s + 1 < n) load_kq(t + 1, kx, qx);
-        const float gd = decay[t * H + h], bt = beta[t * H + h];
-        const float ve = col ? vv[(t * H + h) * (long)E + e] : 0.f;
-        float dot = 0.f;
+    auto stash = [&](const float* reg, float* buf) {
 #pragma unroll
-        for (int i = 0; i < NR; ++i) dot += S[i] * kc[i];
-        dot += __shfl_xor(dot, 1, kWave);
-        dot += __shfl_xor(dot, 2, kWave);
-        const float u = bt * (ve - gd * dot);
-        float out = 0.f;
-#pragma unroll
-        for (int i = 0; i < NR; ++i) {
-            S[i] = gd * S[i] + kc[i] * u;
-            out += S[i] * qc[i];
+        for (int x = 0; x < NLD; ++x) {
+            const int j = tid + x * 256;
+            if (j < 2 * CT * 4 * NR) {
+                const int which = j / (CT * 4 * NR), jj = j - which * (CT * 4 * NR);
+                const int tok = jj / (4 * NR), d = jj - tok * (4 * NR);
+                buf[which * KQ + (tok * 4 + d / NR) * RS + d % NR] = reg[x];
+            } else if (j < 2 * CT * 4 * NR + CT * 64 + 2 * CT) {
+                buf[2 * KQ + j - 2 * CT * 4 * NR] = reg[x];
+            }
         }
-        out += __shfl_xor(out, 1, kWave);
-        out += __shfl_xor(out, 2, kWave);
-        if (col && r == 0) o[(t * H + h) * (long)E + e] = out;
-        if (s + 1 < n) {
+    };
+    float reg[NLD];
+    fetch(0, reg);
+    stash(reg, sm);
+    __syncthreads();
+    const int nchunks = (n + CT - 1) / CT;
+    for (int ch = 0; ch < nchunks; ++ch) {
+        const float* buf = sm + (ch & 1) * BUF;
+        if (ch + 1 < nchunks) fetch(ch + 1, reg);
+        const int nt = min(CT, n - ch * CT);
+        for (int tok = 0; tok < nt; ++tok) {
+            const float4* kp = reinterpret_cast<const float4*>(buf + (tok * 4 + r) * RS);
+            const float4* qp = reinterpret_cast<const float4*>(buf + KQ + (tok * 4 + r) * RS);
+            const float ve = buf[2 * KQ + tok * 64 + c];
+            const float bt = buf[2 * KQ + CT * 64 + tok], gd = buf[2 * KQ + CT * 64 + CT + tok];
+            float kc[NR];
+            float dot = 0.f;
 #pragma unroll
-            for (int i = 0; i < NR; ++i) { kc[i] = kx[i]; qc[i] = qx[i]; }
+            for (int i = 0; i < NR / 4; ++i) {
+                const float4 k4 = kp[i];
+                kc[4 * i] = k4.x; kc[4 * i + 1] = k4.y; kc[4 * i + 2] = k4.z; kc[4 * i + 3] = k4.w;
+            }
+#pragma unroll
+            for (int i = 0; i < NR; ++i) dot += S[i] * kc[i];
+            dot += __shfl_xor(dot, 1, kWave);
+            dot += __shfl_xor(dot, 2, kWave);
+            const float u = bt * (ve - gd * dot);
+            float out = 0.f;
+#pragma unroll
+            for (int i = 0; i < NR / 4; ++i) {
+                const float4 q4 = qp[i];
+                S[4 * i] = gd * S[4 * i] + kc[4 * i] * u;             out += S[4 * i] * q4.x;
+                S[4 * i + 1] = gd * S[4 * i + 1] + kc[4 * i + 1] * u; out += S[4 * i + 1] * q4.y;
+                S[4 * i + 2] = gd * S[4 * i + 2] + kc[4 * i + 2] * u; out += S[4 * i + 2] * q4.z;
+                S[4 * i + 3] = gd * S[4 * i + 3] + kc[4 * i + 3] * u; out += S[4 * i + 3] * q4.w;
+            }
+            out += __shfl_xor(out, 1, kWave);
+            out += __shfl_xor(out, 2, kWave);
+            if (col && r == 0) o[((first + ch * CT + tok) * H + h) * (long)E + e] = out;
         }
+        if (ch + 1 < nchunks) stash(reg, sm + ((ch + 1) & 1) * BUF);
+        __syncthreads();
     }
     if (col) {
 #pragma unroll
         for (int i = 0; i < NR; ++i)
             if (d0 + i < D) sp[(long)(d0 + i) * E] = S[i];
     }
+}
+
+template <int NR>
+static void launch_scan(dim3 grid, hipStream_t s, const void* qn, const void* kn, const void* vv,
+                        const void* beta, const void* decay, void* state, const void* cu_q,
+                        const void* positions, const void* slots, void* o, int H, int G, int D, int E) {
+    constexpr int CT = ScanChunk<NR>::tokens;
+    constexpr int BUF = 2 * CT * 4 * (NR + 4) + CT * 64 + 2 * CT;
+    hipLaunchKernelGGL(delta_scan_kernel<NR>, grid, dim3(256), 2 * BUF * sizeof(float), s,
+                       (const float*)qn, (const float*)kn, (const float*)vv, (const float*)beta,
+                       (const float*)decay, (float*)state, (const int*)cu_q, (const int*)positions,
+                       (const int*)slots, (float*)o, H, G, D, E);
 }
 
 extern "C" {
@@ -208,18 +273,13 @@ int hyb_delta_scan(const void* qn, const void* kn, const void* vv, const void* b
                    const void* decay, void* state, const void* cu_q, const void* positions,
                    const void* slots, void* o, int B, int H, int G, int D, int E, hipStream_t s) {
     if (B <= 0) return 0;
-    if (H % G || D > 512) return 1;
-    const dim3 grid(B, H, (E + 63) / 64), block(256);
-#define SCAN(NR)                                                                              \
-    hipLaunchKernelGGL(delta_scan_kernel<NR>, grid, block, 0, s, (const float*)qn,            \
-                       (const float*)kn, (const float*)vv, (const float*)beta,                \
-                       (const float*)decay, (float*)state, (const int*)cu_q,                  \
-                       (const int*)positions, (const int*)slots, (float*)o, H, G, D, E)
+    if (H % G || D > 256) return 1;
+    const dim3 grid(B, H, (E + 63) / 64);
+#define SCAN(NR) launch_scan<NR>(grid, s, qn, kn, vv, beta, decay, state, cu_q, positions, slots, o, H, G, D, E)
     if (D <= 32) SCAN(8);
     else if (D <= 64) SCAN(16);
     else if (D <= 128) SCAN(32);
-    else if (D <= 256) SCAN(64);
-    else SCAN(128);
+    else SCAN(64);
 #undef SCAN
     return HYB_LAUNCH_OK();
 }

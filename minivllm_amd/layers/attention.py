@@ -188,16 +188,15 @@ class SinkAttention(nn.Module):
         if not ctx.is_prefill:
             ops.sink_attention_decode(q, *a, ctx.block_tables, ctx.context_lens, self.scale,
                                       self.sink, gate, out)
-        elif q.is_cuda:
-            # one launch for every row of the step, decode riders included: a row's context is
-            # its position + 1 keys of its sequence
-            ops.sink_attention_step(q, *a, ctx.block_tables, ctx.row_seq, ctx.positions,
-                                    self.scale, self.sink, gate, out)
         else:
+            # prompt portions through the prefill kernel, the single next tokens that ride along
+            # (the first num_decode_seqs rows and sequences) through the decode kernel
             Bd = ctx.num_decode_seqs
             if ctx.num_seqs > Bd:
                 ops.sink_attention_prefill(q, *a, ctx.cu_seqlens_q[Bd:], ctx.cu_seqlens_k[Bd:],
-                                           ctx.block_tables[Bd:], self.scale, self.sink, gate, out)
+                                           ctx.block_tables[Bd:], self.scale, self.sink, gate, out,
+                                           positions=ctx.positions, max_q=ctx.max_seqlen_q or None,
+                                           row_seq=ctx.row_seq, first_seq=Bd)
             if Bd:
                 ops.sink_attention_decode(q[:Bd], *a, ctx.block_tables[:Bd], ctx.context_lens,
                                           self.scale, self.sink,

@@ -262,9 +262,18 @@ def pair_rope_mix_store(q, k, v, positions, cos_sin, rot_dims, v_first, lam, v_m
                                           v_mode, k_cache, v_cache, slot_mapping)
 
 
-def sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables, scale, sink, gate, out):
-    return _seqmix(q).sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables,
-                                             scale, sink, gate, out)
+def sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables, scale, sink, gate, out,
+                           positions=None, max_q=None, row_seq=None, first_seq=0):
+    """``positions`` [T], ``max_q`` (longest portion, a host integer), ``row_seq`` and ``first_seq``
+    (how many sequences of the step precede ``cu_q[0]``'s, i.e. what was sliced off): what the
+    GPU kernels take besides (``hip_hybrid.sink_attention_prefill``); the CPU form derives
+    everything from ``cu_q`` / ``cu_k``."""
+    if _on_gpu(q):
+        return _hybrid().sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables,
+                                                scale, sink, gate, out, positions=positions,
+                                                max_q=max_q, row_seq=row_seq, first_seq=first_seq)
+    return torch_seqmix.sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables,
+                                               scale, sink, gate, out)
 
 
 def sink_attention_step(q, k_cache, v_cache, block_tables, row_seq, positions, scale, sink, gate,

@@ -39,7 +39,12 @@ _ghn = _sig("hyb_gated_head_norm", _P, _P, _P, _L, _P, _L, _I, _I, _F, _I, _P)
 _route = _sig("hyb_grouped_route", _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _P)
 _gelu = _sig("hyb_gelu_route_scale", _P, _P, _P, _L, _I, _I, _I, _P)
 _attn = _sig("hyb_sink_attention_rows", _P, _L, _L, _P, _P, _P, _I, _I, _P, _P, _I, _P, _P, _L, _P,
-             _F, _L, _I, _I, _I, _I, _I, _P)
+             _F, _L, _I, _I, _I, _I, _I, _I, _P)
+_tiles = _sig("hyb_sink_attention_tiles", _P, _L, _L, _P, _P, _P, _I, _I, _P, _P, _P, _P, _L, _P, _F,
+              _I, _I, _I, _I, _I, _I, _I, _I, _P)
+_tiles_ok = _lib.hyb_sink_attention_tiles_ok
+_tiles_ok.argtypes = [_I, _I]
+_tiles_ok.restype = _I
 _prep = _sig("hyb_delta_prepare", _P, _L, _I, _I, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P,
              _P, _P, _L, _I, _I, _I, _I, _I, _I, _P)
 _scan = _sig("hyb_delta_scan", _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P)
@@ -138,7 +143,8 @@ def pair_rope_mix_store(q, k, v, positions, cos_sin, rot_dims, v_first, lam, v_m
 
 
 # ------------------------------------------------------------------ attention with a sink
-def _attention_rows(q, k_cache, v_cache, block_tables, row_seq, lens, len_add, scale, sink, gate, out):
+def _attention_rows(q, k_cache, v_cache, block_tables, row_seq, lens, len_add, scale, sink, gate, out,
+                    seq_base=0):
     T, H, D = q.shape
     G, E = k_cache.shape[2], v_cache.shape[3]
     assert q.stride(2) == 1 and out.is_contiguous() and out.shape == (T, H, E) and out.dtype == q.dtype
@@ -150,15 +156,52 @@ def _attention_rows(q, k_cache, v_cache, block_tables, row_seq, lens, len_add, s
                  block_tables.data_ptr(), block_tables.stride(0), k_cache.shape[1],
                  _ptr(_i32(row_seq)), _i32(lens).data_ptr(), len_add, _f32(sink).data_ptr(),
                  _ptr(gate), gate.stride(0) if gate is not None else 0, out.data_ptr(), scale, T,
-                 H, G, D, E, _dt(q), _stream()), "sink_attention")
+                 H, G, D, E, seq_base, _dt(q), _stream()), "sink_attention")
     return out
 
 
-def sink_attention_step(q, k_cache, v_cache, block_tables, row_seq, positions, scale, sink, gate, out):
-    """Every row of a prefill-form step (portions of prompts and single next tokens alike): row
-    t belongs to sequence ``row_seq[t]`` (< 0: none) and sees ``positions[t] + 1`` keys."""
+def sink_attention_step(q, k_cache, v_cache, block_tables, row_seq, positions, scale, sink, gate, out,
+                        seq_base=0):
+    """Rows of a prefill-form step, one workgroup per row: row t belongs to sequence
+    ``row_seq[t]`` (< ``seq_base``: skipped), whose block table is row ``row_seq[t] - seq_base``
+    of ``block_tables``, and sees ``positions[t] + 1`` keys."""
     return _attention_rows(q, k_cache, v_cache, block_tables, row_seq, positions, 1, scale, sink,
-                           gate, out)
+                           gate, out, seq_base)
+
+
+def sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables, scale, sink, gate, out,
+                           positions=None, max_q=None, row_seq=None, first_seq=0):
+    """The prompt portions of a step: sequence b owns rows cu_q[b] .. cu_q[b+1] (absolute rows
+    of q / out / positions) and block table row b.  Runs the matrix-core tile kernel (fp32
+    scores, weights and sums); head sizes it has no instance for go row by row.  ``cu_k`` is
+    not needed (a row's context is its position + 1)."""
+    T, H, D = q.shape
+    G, E = k_cache.shape[2], v_cache.shape[3]
+    nseq = cu_q.shape[0] - 1
+    assert positions is not None, "the GPU form takes the rows' positions"
+    if not _tiles_ok(D, E):
+        assert row_seq is not None
+        # ``first_seq``: number of the step's sequences ahead of these (its decode riders)
+        return sink_attention_step(q, k_cache, v_cache, block_tables, row_seq, positions, scale,
+                                   sink, gate, out, seq_base=first_seq)
+    if max_q is None:
+        max_q = int((cu_q[1:] - cu_q[:-1]).max())
+    assert q.stride(2) == 1 and out.is_contiguous() and out.shape == (T, H, E) and out.dtype == q.dtype
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dtype == q.dtype
+    assert block_tables.dtype == torch.int32 and block_tables.stride(1) == 1
+    if gate is not None:
+        assert gate.stride(1) == 1 and gate.dtype == q.dtype
+    _check(_tiles(q.data_ptr(), q.stride(0), q.stride(1), k_cache.data_ptr(), v_cache.data_ptr(),
+                  block_tables.data_ptr(), block_tables.stride(0), k_cache.shape[1],
+                  _i32c(cu_q).data_ptr(), _i32(positions).data_ptr(), _f32(sink).data_ptr(),
+                  _ptr(gate), gate.stride(0) if gate is not None else 0, out.data_ptr(), scale,
+                  nseq, 0, max_q, H, G, D, E, _dt(q), _stream()), "sink_attention_prefill")
+    return out
+
+
+def _i32c(t):
+    assert t.dtype == torch.int32 and t.stride(0) == 1
+    return t
 
 
 def sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens, scale, sink, gate, out):

@@ -103,7 +103,8 @@ def weights(c, seed=0, qk_gain=3.0):
         elif name in ("embed", "bigram"):
             t = r
         else:
-            t = r * shape[-1] ** -0.5 * (qk_gain if leaf in ("q", "k", "router") else 1.0)
+            gain = qk_gain if leaf in ("q", "k") else 2 * qk_gain if leaf == "router" else 1.0
+            t = r * shape[-1] ** -0.5 * gain
         out[name] = t.to(torch.bfloat16)
     return out
 

@@ -146,17 +146,18 @@ def grouped_top_experts(z: torch.Tensor, top: int, groups: int, keep: int):
 
 
 def routing_margin(z: torch.Tensor, top: int, groups: int, keep: int) -> float:
-    """How far the routing decision for logits z is from flipping: the smallest gap between a
-    kept and a dropped group's best score, or between a chosen and an eligible unchosen score."""
-    s = torch.softmax(z, -1)
-    per = s.shape[0] // groups
-    best = s.view(groups, per).max(-1).values.sort(descending=True).values
-    m = float(best[keep - 1] - best[keep]) if keep < groups else 1.0
+    """How far the routing decision for logits z is from flipping, in logit units: the smallest
+    gap between a kept and a dropped group's best logit, or between a chosen and an eligible
+    unchosen logit (scores are a monotone function of the logits)."""
+    per = z.shape[0] // groups
+    gbest = z.view(groups, per).max(-1).values
+    best = gbest.sort(descending=True).values
+    m = float(best[keep - 1] - best[keep]) if keep < groups else float("inf")
     ids, _ = grouped_top_experts(z, top, groups, keep)
-    kept = torch.topk(s.view(groups, per).max(-1).values, keep).indices.tolist()
-    rest = [float(s[e]) for gi in kept for e in range(gi * per, (gi + 1) * per) if e not in ids]
+    kept = torch.topk(gbest, keep).indices.tolist()
+    rest = [float(z[e]) for gi in kept for e in range(gi * per, (gi + 1) * per) if e not in ids]
     if rest:
-        m = min(m, float(s[ids].min()) - max(rest))
+        m = min(m, float(z[ids].min()) - max(rest))
     return m
 
 
@@ -242,7 +243,7 @@ class Oracle:
         pos = torch.arange(st["n"], st["n"] + T)
         shared = {}
         self.trace = []
-        self.margin = [1.0] * T          # per token: the closest routing decision of any layer
+        self.margin = [float('inf')] * T          # per token: the closest routing decision of any layer
         for i, layer in enumerate(cfg["layers"]):
             p, ls, m = f"l{i}.", st["layers"][i], layer["mixer"]
             h = norm_around_zero(x, w[p + "norm1"], self.eps)

@@ -52,7 +52,7 @@ def close(got, want, dtype):
     # and stores, so there the bound is what rounding does to these small, high-gain models
     # (a peaked softmax or a routing weight amplifies single roundings): typical rows tight,
     # the worst row loose
-    lim = 2e-4 if dtype == "float32" else 0.12
+    lim = 2e-4 if dtype == "float32" else 0.25
     assert float(e.max()) < lim, f"logits differ: {float(e.max()):.3g} (limit {lim})"
     if dtype != "float32":
         assert float(e.median()) < 0.04, f"typical row differs: {float(e.median()):.3g}"
@@ -84,7 +84,7 @@ class Expected:
     def __init__(self, c, w, toks):
         o = Oracle(c, w)
         self.logits = o.feed(toks).float()
-        close_calls = [t for t, m in enumerate(o.margin) if m < 0.03]
+        close_calls = [t for t, m in enumerate(o.margin) if m < 0.08]
         self.sure = close_calls[0] if close_calls else len(toks)
         self.trace = o.trace
 
@@ -105,6 +105,7 @@ def test_whole_prompt_and_every_layer(tmp_path, device, dtype):
     close(got, want, dtype)
     assert len(seen) == len(c["layers"])
     n = len(toks) if dtype == "float32" else want.sure
+    assert n >= 10, "the fixture's routing is a close call too early for a 16-bit comparison"
     for x, ref in zip(seen, want.trace):
         lim = 1e-4 if dtype == "float32" else 0.15
         assert float((x[:n] - ref.float()[:n]).abs().max()) < lim * float(ref.abs().max())

@@ -116,6 +116,45 @@ def test_sink_attention_decode_and_step(dt, H, G, D, E):
     og = hk.sink_attention_step(*dev(q, kc, vc, tables, row_seq, pos), 0.3, sink.cuda(), gate.cuda(),
                                 torch.zeros(T, H, E, dtype=dt).cuda())
     torch.testing.assert_close(og.cpu().float(), o.float(), **tol(dt))
+    # the prompt-portion entry point (matrix-core tiles where the head sizes have an instance)
+    og = hk.sink_attention_prefill(*dev(q, kc, vc, cu_q, cu_k, tables), 0.3, sink.cuda(), gate.cuda(),
+                                   torch.zeros(T, H, E, dtype=dt).cuda(), positions=pos.cuda(),
+                                   max_q=max(qlens), row_seq=row_seq.cuda())
+    torch.testing.assert_close(og.cpu().float(), o.float(), **tol(dt))
+    # ... and behind two sequences that are sliced off (a mixed step's decode riders)
+    og = hk.sink_attention_prefill(*dev(q, kc, vc, cu_q[2:], cu_k[2:], tables[2:]), 0.3, sink.cuda(),
+                                   gate.cuda(), torch.zeros(T, H, E, dtype=dt).cuda(),
+                                   positions=pos.cuda(), max_q=max(qlens[2:]), row_seq=row_seq.cuda(),
+                                   first_seq=2)
+    lo = int(cu_q[2])
+    torch.testing.assert_close(og.cpu().float()[lo:int(cu_q[-1])], o.float()[lo:int(cu_q[-1])], **tol(dt))
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("H,G,D,E", [(2, 1, 128, 128), (4, 2, 64, 256), (2, 2, 200, 72), (2, 1, 260, 8)])
+def test_sink_attention_prefill_long_portions(dt, H, G, D, E):
+    """Portions longer than a workgroup's 128 queries, contexts that end inside a key tile,
+    head sizes of every template instance and one (D > 256) that goes row by row."""
+    torch.manual_seed(6)
+    bs = 32
+    lens, qlens = [700, 131, 33], [300, 131, 1]
+    kc, vc, tables = _paged(lens, bs, G, D, E, dt)
+    kc, vc = 0.3 * kc, vc
+    cu_q = torch.tensor([0] + list(torch.tensor(qlens).cumsum(0)), dtype=torch.int32)
+    cu_k = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    T = int(cu_q[-1])
+    q, gate, sink = torch.randn(T, H, D).to(dt), torch.randn(T, H).to(dt), torch.randn(H)
+    row_seq = torch.zeros(T, dtype=torch.int32)
+    pos = torch.zeros(T, dtype=torch.int32)
+    for b, (n, L) in enumerate(zip(qlens, lens)):
+        row_seq[cu_q[b]:cu_q[b + 1]] = b
+        pos[cu_q[b]:cu_q[b + 1]] = torch.arange(L - n, L, dtype=torch.int32)
+    o = ref.sink_attention_prefill(q, kc, vc, cu_q, cu_k, tables, D ** -0.5, sink, gate,
+                                   torch.zeros(T, H, E, dtype=dt))
+    og = hk.sink_attention_prefill(*dev(q, kc, vc, cu_q, cu_k, tables), D ** -0.5, sink.cuda(), gate.cuda(),
+                                   torch.zeros(T, H, E, dtype=dt).cuda(), positions=pos.cuda(),
+                                   max_q=max(qlens), row_seq=row_seq.cuda())
+    torch.testing.assert_close(og.cpu().float(), o.float(), **tol(dt))
 
 
 def test_sink_decides_when_scores_are_low():
