@@ -353,7 +353,186 @@ static int launch_tiles(const void* q, long q_row, long q_head, const void* k_ca
     return HYB_LAUNCH_OK();
 }
 
+// ---------------------------------------------------------------------------------------
+// Decode rows at serving sizes: the context is split over workgroups and every K / V row is
+// read by 16 neighbouring lanes with 16-byte (bf16: EPL = 8 elements) loads, so a wave streams
+// four whole rows per step.  A 16-lane group walks its own keys (group kg of 16 per workgroup,
+// keys kg, kg + 16, ...) with a private running softmax for up to 4 query heads of the KV head;
+// the groups' partials meet in LDS, the workgroups' (one per context split) in a workspace that
+// `sink_attention_merge_kernel` folds together with the sink term and the gate.
+// EPL / VPL: elements of a K / V row per lane (D = 16 EPL, E = 16 VPL).
+template <typename T, int N> __device__ __forceinline__ void load_run(const T* p, float* o) {
+#pragma unroll
+    for (int i = 0; i < N; i += 4) Vec4<T>::load(p + i, o + i);
+}
+
+template <typename T, int EPL, int VPL>
+__global__ void __launch_bounds__(256)
+sink_attention_split_kernel(const T* __restrict__ q, long q_row, long q_head,
+                            const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+                            const int* __restrict__ block_tables, int max_blocks, int block_size,
+                            const int* __restrict__ context_lens, const float* __restrict__ sink,
+                            float* __restrict__ ws, float scale, int H, int G, int splits) {
+    constexpr int D = 16 * EPL, E = 16 * VPL;
+    extern __shared__ float sm[];                 // [16 groups][RC][E + 2]
+    const int R = H / G, chunks = (R + RC - 1) / RC;
+    const int b = blockIdx.x, split = blockIdx.z;
+    const int g = blockIdx.y / chunks, h0 = g * R + (blockIdx.y % chunks) * RC;
+    const int nr = min(RC, g * R + R - h0);
+    const int ctx = context_lens[b];
+    const int tid = threadIdx.x, lane16 = tid & 15, kg = tid >> 4;
+    const int span = ((ctx + splits - 1) / splits + 15) & ~15;
+    const int k_begin = split * span, k_end = min(ctx, k_begin + span);
+    const int* table = block_tables + (long)b * max_blocks;
+
+    float qf[RC][EPL], m[RC], l[RC], acc[RC][VPL];
+#pragma unroll
+    for (int r = 0; r < RC; ++r) {
+        if (r < nr) {
+            load_run<T, EPL>(q + b * q_row + (long)(h0 + r) * q_head + lane16 * EPL, qf[r]);
+#pragma unroll
+            for (int i = 0; i < EPL; ++i) qf[r][i] *= scale;
+            m[r] = sink[h0 + r];
+        } else {
+#pragma unroll
+            for (int i = 0; i < EPL; ++i) qf[r][i] = 0.f;
+            m[r] = 0.f;
+        }
+        l[r] = 0.f;
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) acc[r][i] = 0.f;
+    }
+    for (int j = k_begin + kg; j < k_end; j += 16) {
+        const long slot = (long)table[j / block_size] * block_size + j % block_size;
+        float kf[EPL], vf[VPL];
+        load_run<T, EPL>(k_cache + (slot * G + g) * (long)D + lane16 * EPL, kf);
+        load_run<T, VPL>(v_cache + (slot * G + g) * (long)E + lane16 * VPL, vf);
+#pragma unroll
+        for (int r = 0; r < RC; ++r) {
+            if (r >= nr) continue;
+            float d = 0.f;
+#pragma unroll
+            for (int i = 0; i < EPL; ++i) d += kf[i] * qf[r][i];
+            d += __shfl_xor(d, 1, kWave);
+            d += __shfl_xor(d, 2, kWave);
+            d += __shfl_xor(d, 4, kWave);
+            d += __shfl_xor(d, 8, kWave);
+            if (d > m[r]) {                        // the running maximum moves: rescale (rare)
+                const float a = expf(m[r] - d);
+                l[r] *= a;
+#pragma unroll
+                for (int i = 0; i < VPL; ++i) acc[r][i] *= a;
+                m[r] = d;
+            }
+            const float p = expf(d - m[r]);
+            l[r] += p;
+#pragma unroll
+            for (int i = 0; i < VPL; ++i) acc[r][i] += p * vf[i];
+        }
+    }
+    // the 16 groups' partials -> LDS -> one partial per (head, split)
+    constexpr int PS = E + 2;
+#pragma unroll
+    for (int r = 0; r < RC; ++r) {
+        float* dst = sm + (kg * RC + r) * PS;
+        if (lane16 == 0) { dst[0] = m[r]; dst[1] = l[r]; }
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) dst[2 + lane16 * VPL + i] = acc[r][i];
+    }
+    __syncthreads();
+    for (int c = tid; c < nr * PS; c += 256) {
+        const int r = c / PS, x = c - r * PS;
+        float M = sm[r * PS];
+        for (int k = 1; k < 16; ++k) M = fmaxf(M, sm[(k * RC + r) * PS]);
+        float v;
+        if (x == 0) v = M;
+        else {
+            v = 0.f;
+            for (int k = 0; k < 16; ++k) {
+                const float* src = sm + (k * RC + r) * PS;
+                v += src[x] * expf(src[0] - M);
+            }
+        }
+        ws[(((long)b * H + h0 + r) * splits + split) * PS + x] = v;
+    }
+}
+
+template <typename T>
+__global__ void sink_attention_merge_kernel(const float* __restrict__ ws,
+                                            const float* __restrict__ sink,
+                                            const T* __restrict__ gate, long gate_row,
+                                            const int* __restrict__ context_lens,
+                                            T* __restrict__ out, int H, int E, int splits) {
+    const int b = blockIdx.x / H, h = blockIdx.x % H;
+    if (context_lens[b] <= 0) return;
+    const int PS = E + 2;
+    const float* p = ws + ((long)b * H + h) * splits * PS;
+    float M = sink[h];
+    for (int s = 0; s < splits; ++s) M = fmaxf(M, p[s * PS]);
+    float L = expf(sink[h] - M);
+    for (int s = 0; s < splits; ++s) L += p[s * PS + 1] * expf(p[s * PS] - M);
+    float f = 1.f / L;
+    if (gate) f *= sigmoidf_(ld(gate + b * gate_row + h));
+    for (int e = threadIdx.x; e < E; e += blockDim.x) {
+        float v = 0.f;
+        for (int s = 0; s < splits; ++s) v += p[s * PS + 2 + e] * expf(p[s * PS] - M);
+        st(out + ((long)b * H + h) * E + e, v * f);
+    }
+}
+
+template <typename T, int EPL, int VPL>
+static int launch_split(const void* q, long q_row, long q_head, const void* k_cache,
+                        const void* v_cache, const void* block_tables, int max_blocks,
+                        int block_size, const void* context_lens, const void* sink,
+                        const void* gate, long gate_row, void* out, void* ws, float scale, int B,
+                        int H, int G, int splits, hipStream_t s) {
+    constexpr int E = 16 * VPL;
+    const int R = H / G, chunks = (R + RC - 1) / RC;
+    const size_t lds = 16 * RC * (E + 2) * sizeof(float);
+    hipLaunchKernelGGL((sink_attention_split_kernel<T, EPL, VPL>), dim3(B, G * chunks, splits),
+                       dim3(256), lds, s, (const T*)q, q_row, q_head, (const T*)k_cache,
+                       (const T*)v_cache, (const int*)block_tables, max_blocks, block_size,
+                       (const int*)context_lens, (const float*)sink, (float*)ws, scale, H, G, splits);
+    if (hipGetLastError() != hipSuccess) return 2;
+    hipLaunchKernelGGL(sink_attention_merge_kernel<T>, dim3(B * H), dim3(E >= 128 ? 128 : 64), 0, s,
+                       (const float*)ws, (const float*)sink, (const T*)gate, gate_row,
+                       (const int*)context_lens, (T*)out, H, E, splits);
+    return HYB_LAUNCH_OK();
+}
+
 extern "C" {
+
+// 1 when the split decode kernel has an instance for these head sizes
+int hyb_sink_attention_split_ok(int D, int E) {
+    return (D == 64 || D == 128 || D == 256) && (E == 64 || E == 128);
+}
+
+// Decode rows (row b = sequence b); ws: fp32 workspace of B * H * splits * (E + 2) floats.
+int hyb_sink_attention_split(const void* q, long q_row, long q_head, const void* k_cache,
+                             const void* v_cache, const void* block_tables, int max_blocks,
+                             int block_size, const void* context_lens, const void* sink,
+                             const void* gate, long gate_row, void* out, void* ws, float scale,
+                             int B, int H, int G, int D, int E, int splits, int dt, hipStream_t s) {
+    if (B <= 0) return 0;
+    if (G <= 0 || H % G || splits < 1 || !hyb_sink_attention_split_ok(D, E)) return 1;
+    if (((size_t)k_cache | (size_t)v_cache | (size_t)q) % 16 || (q_row * (dt == 0 ? 2 : 4)) % 16) return 1;
+#define SPLIT_ARGS q, q_row, q_head, k_cache, v_cache, block_tables, max_blocks, block_size, \
+                   context_lens, sink, gate, gate_row, out, ws, scale, B, H, G, splits, s
+#define SPLIT_E(T, EPL)                                                  \
+    do {                                                                 \
+        if (E == 64) return launch_split<T, EPL, 4>(SPLIT_ARGS);         \
+        return launch_split<T, EPL, 8>(SPLIT_ARGS);                      \
+    } while (0)
+#define SPLIT_D(T)                             \
+    do {                                       \
+        if (D == 64) SPLIT_E(T, 4);            \
+        else if (D == 128) SPLIT_E(T, 8);      \
+        else SPLIT_E(T, 16);                   \
+    } while (0)
+    if (dt == 0) SPLIT_D(hyb::bf16_t);
+    else if (dt == 2) SPLIT_D(float);
+    return 1;
+}
 
 // 1 when the tile kernel has an instance for these head sizes (else the row kernel serves)
 int hyb_sink_attention_tiles_ok(int D, int E) { return D <= 256 && E <= 256 && !(D > 128 && E > 128); }

@@ -85,7 +85,7 @@ __global__ void delta_conv_tail_kernel(const T* __restrict__ proj, long row_stri
     if (n <= 0) return;
     const bool has_past = positions[first] > 0;
     float* tail = conv_state + (long)slot * (taps - 1) * C;
-    for (int c = threadIdx.x; c < C; c += blockDim.x) {
+    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < C; c += gridDim.y * blockDim.x) {
         float nv[MAX_TAPS];
 #pragma unroll
         for (int j = 0; j < MAX_TAPS - 1; ++j) {
@@ -252,7 +252,8 @@ int hyb_delta_prepare(const void* proj, long row_stride, int b_off, int a_off, c
     const int C = 2 * G * D + H * E;
     const size_t lds = 2 * (size_t)G * D * sizeof(float);
     if (lds > 64 * 1024) return 1;
-    HYB_DISPATCH(dt, hipLaunchKernelGGL(delta_prepare_kernel<T>, dim3(T_), dim3(256), lds, s,
+    HYB_DISPATCH(dt, hipLaunchKernelGGL(delta_prepare_kernel<T>, dim3(T_), dim3(C >= 2048 && T_ <= 1024 ? 1024 : 256),
+                                        lds, s,
                                         (const T*)proj, row_stride, b_off, a_off,
                                         (const float*)conv_w, taps, (const float*)a_log,
                                         (const float*)dt_bias, (const float*)conv_state,
@@ -261,7 +262,8 @@ int hyb_delta_prepare(const void* proj, long row_stride, int b_off, int a_off, c
                                         (float*)beta, (float*)decay, H, G, D, E));
     if (hipGetLastError() != hipSuccess) return 2;
     if (taps > 1) {
-        HYB_DISPATCH(dt, hipLaunchKernelGGL(delta_conv_tail_kernel<T>, dim3(B), dim3(256), 0, s,
+        HYB_DISPATCH(dt, hipLaunchKernelGGL(delta_conv_tail_kernel<T>, dim3(B, (C + 255) / 256),
+                                            dim3(256), 0, s,
                                             (const T*)proj, row_stride, taps, (float*)conv_state,
                                             (const int*)cu_q, (const int*)positions,
                                             (const int*)slots, C));

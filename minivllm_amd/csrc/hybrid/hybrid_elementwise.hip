@@ -125,9 +125,10 @@ __global__ void gated_head_norm_kernel(const float* __restrict__ o, const float*
         st(out + th * E + e, orow[e] * r * w[e] * siluf_(ld(g + e)));
 }
 
-// One wave per token: fp32 router logits, softmax over all experts, best `keep` of `groups`
-// groups (a group scores its best expert), `top` largest eligible scores; dense [T, NE] out,
-// zero where not chosen.  Ties go to the lower index.  LDS: 2 * NE floats.
+// One workgroup (256 threads) per token: fp32 router logits (the row is read once, eight experts'
+// partial sums per pass), softmax over all experts, best `keep` of `groups` groups (a group
+// scores its best expert), `top` largest eligible scores; dense [T, NE] out, zero where not
+// chosen.  Ties go to the lower index.  LDS: 2 * NE + 32 floats.
 template <typename T>
 __global__ void grouped_route_kernel(const T* __restrict__ h, const float* __restrict__ wr,
                                      float* __restrict__ dense, int W, int NE, int top,
@@ -135,24 +136,48 @@ __global__ void grouped_route_kernel(const T* __restrict__ h, const float* __res
     extern __shared__ float sm[];
     float* z = sm;              // scores
     float* elig = sm + NE;      // eligible scores (or -1)
+    float* red = sm + 2 * NE;   // [4 waves][8]
     const long t = blockIdx.x;
     const T* hr = h + t * W;
-    for (int e = 0; e < NE; ++e) {
-        float s = 0.f;
-        for (int c = threadIdx.x; c < W; c += kWave) s += ld(hr + c) * wr[(long)e * W + c];
-        s = wave_sum(s);
-        if (threadIdx.x == 0) z[e] = s;
+    for (int e0 = 0; e0 < NE; e0 += 8) {
+        float acc[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+#pragma unroll 4
+        for (int c = threadIdx.x; c < W; c += blockDim.x) {
+            const float hv = ld(hr + c);
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if (e0 + j < NE) acc[j] += hv * wr[(long)(e0 + j) * W + c];
+        }
+        // eight sums at once: per wave by exchanges, across the 4 waves through LDS
+        const int wave = threadIdx.x / kWave, nw = blockDim.x / kWave;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float sj = wave_sum(acc[j]);
+            if ((threadIdx.x & (kWave - 1)) == 0) red[wave * 8 + j] = sj;
+        }
+        __syncthreads();
+        if (threadIdx.x < 8 && e0 + threadIdx.x < NE) {
+            float sj = 0.f;
+            for (int w = 0; w < nw; ++w) sj += red[w * 8 + threadIdx.x];
+            z[e0 + threadIdx.x] = sj;
+        }
+        __syncthreads();
     }
-    __syncthreads();
-    float m = -INFINITY;
-    for (int e = threadIdx.x; e < NE; e += kWave) m = fmaxf(m, z[e]);
-    m = wave_max(m);
-    float sum = 0.f;
-    for (int e = threadIdx.x; e < NE; e += kWave) sum += expf(z[e] - m);
-    sum = wave_sum(sum);
-    __syncthreads();
-    for (int e = threadIdx.x; e < NE; e += kWave) { z[e] = expf(z[e] - m) / sum; elig[e] = -1.f; }
-    for (int e = threadIdx.x; e < NE; e += kWave) dense[t * NE + e] = 0.f;
+    if (threadIdx.x < kWave) {
+        float m = -INFINITY;
+        for (int e = threadIdx.x; e < NE; e += kWave) m = fmaxf(m, z[e]);
+        m = wave_max(m);
+        float sum = 0.f;
+        for (int e = threadIdx.x; e < NE; e += kWave) sum += expf(z[e] - m);
+        sum = wave_sum(sum);
+        for (int e = threadIdx.x; e < NE; e += kWave) {
+            z[e] = expf(z[e] - m) / sum;
+            elig[e] = -1.f;
+            dense[t * NE + e] = 0.f;
+        }
+    }
     __syncthreads();
     if (threadIdx.x == 0) {
         const int per = NE / groups;
@@ -176,16 +201,27 @@ __global__ void grouped_route_kernel(const T* __restrict__ h, const float* __res
     }
 }
 
-// act[t, e*ff + j] = gelu(up[t, e*ff + j]) * dense[t, e]
-template <typename T>
+// act[t, e*ff + j] = gelu(up[t, e*ff + j]) * dense[t, e]; VEC elements per thread and step (one
+// expert lookup per run; ff % VEC == 0)
+template <typename T, int VEC>
 __global__ void gelu_route_scale_kernel(const T* __restrict__ up, const float* __restrict__ dense,
                                         T* __restrict__ act, long n, int NE, int ff) {
     const long cols = (long)NE * ff;
-    for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+    for (long i = (blockIdx.x * (long)blockDim.x + threadIdx.x) * VEC; i < n;
+         i += (long)gridDim.x * blockDim.x * VEC) {
         const long t = i / cols;
         const int e = (int)((i - t * cols) / ff);
         const float w = dense[t * NE + e];
-        st(act + i, w == 0.f ? 0.f : gelu_erf(ld(up + i)) * w);
+        if (w == 0.f) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) st(act + i + j, 0.f);
+        } else {
+            float v[VEC];
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[j] = ld(up + i + j);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) st(act + i + j, gelu_erf(v[j]) * w);
+        }
     }
 }
 
@@ -247,8 +283,8 @@ int hyb_grouped_route(const void* h, const void* wr, void* dense, long T_, int W
                       int groups, int keep, int dt, hipStream_t s) {
     if (T_ <= 0) return 0;
     if (groups <= 0 || NE % groups || keep > groups || top > NE / groups * keep || NE > 4096) return 1;
-    HYB_DISPATCH(dt, hipLaunchKernelGGL(grouped_route_kernel<T>, dim3(T_), dim3(kWave),
-                                        2 * NE * sizeof(float), s, (const T*)h, (const float*)wr,
+    HYB_DISPATCH(dt, hipLaunchKernelGGL(grouped_route_kernel<T>, dim3(T_), dim3(256),
+                                        (2 * NE + 32) * sizeof(float), s, (const T*)h, (const float*)wr,
                                         (float*)dense, W, NE, top, groups, keep));
     return HYB_LAUNCH_OK();
 }
@@ -257,9 +293,16 @@ int hyb_gelu_route_scale(const void* up, const void* dense, void* act, long T_, 
                          int dt, hipStream_t s) {
     const long n = T_ * NE * ff;
     if (n <= 0) return 0;
-    const int blocks = (int)((n + 255) / 256 > 8192 ? 8192 : (n + 255) / 256);
-    HYB_DISPATCH(dt, hipLaunchKernelGGL(gelu_route_scale_kernel<T>, dim3(blocks), dim3(256), 0, s,
-                                        (const T*)up, (const float*)dense, (T*)act, n, NE, ff));
+    if (ff % 8 == 0) {
+        const long work = n / 8;
+        const int blocks = (int)((work + 255) / 256 > 16384 ? 16384 : (work + 255) / 256);
+        HYB_DISPATCH(dt, hipLaunchKernelGGL((gelu_route_scale_kernel<T, 8>), dim3(blocks), dim3(256),
+                                            0, s, (const T*)up, (const float*)dense, (T*)act, n, NE, ff));
+    } else {
+        const int blocks = (int)((n + 255) / 256 > 16384 ? 16384 : (n + 255) / 256);
+        HYB_DISPATCH(dt, hipLaunchKernelGGL((gelu_route_scale_kernel<T, 1>), dim3(blocks), dim3(256),
+                                            0, s, (const T*)up, (const float*)dense, (T*)act, n, NE, ff));
+    }
     return HYB_LAUNCH_OK();
 }
 

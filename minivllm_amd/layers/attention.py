@@ -187,7 +187,7 @@ class SinkAttention(nn.Module):
         a = (self.k_cache, self.v_cache)
         if not ctx.is_prefill:
             ops.sink_attention_decode(q, *a, ctx.block_tables, ctx.context_lens, self.scale,
-                                      self.sink, gate, out)
+                                      self.sink, gate, out, ctx.max_context_len or None)
         else:
             # prompt portions through the prefill kernel, the single next tokens that ride along
             # (the first num_decode_seqs rows and sequences) through the decode kernel
@@ -200,5 +200,6 @@ class SinkAttention(nn.Module):
             if Bd:
                 ops.sink_attention_decode(q[:Bd], *a, ctx.block_tables[:Bd], ctx.context_lens,
                                           self.scale, self.sink,
-                                          None if gate is None else gate[:Bd], out[:Bd])
+                                          None if gate is None else gate[:Bd], out[:Bd],
+                                          ctx.max_context_len or None)
         return out.view(T, self.num_heads * self.v_head_dim)

@@ -283,9 +283,15 @@ def sink_attention_step(q, k_cache, v_cache, block_tables, row_seq, positions, s
                                          scale, sink, gate, out)
 
 
-def sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens, scale, sink, gate, out):
-    return _seqmix(q).sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens,
-                                            scale, sink, gate, out)
+def sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens, scale, sink, gate, out,
+                          max_context_len=None):
+    """``max_context_len`` (a host integer, an upper bound will do): lets the GPU form size its
+    context splits without reading the lengths back."""
+    if _on_gpu(q):
+        return _hybrid().sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens,
+                                               scale, sink, gate, out, max_context_len)
+    return torch_seqmix.sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens,
+                                              scale, sink, gate, out)
 
 
 def delta_prepare(q, k, v, b, a, conv_w, a_log, dt_bias, conv_state, cu_q, positions, slots,

@@ -45,6 +45,11 @@ _tiles = _sig("hyb_sink_attention_tiles", _P, _L, _L, _P, _P, _P, _I, _I, _P, _P
 _tiles_ok = _lib.hyb_sink_attention_tiles_ok
 _tiles_ok.argtypes = [_I, _I]
 _tiles_ok.restype = _I
+_split = _sig("hyb_sink_attention_split", _P, _L, _L, _P, _P, _P, _I, _I, _P, _P, _P, _L, _P, _P, _F,
+              _I, _I, _I, _I, _I, _I, _I, _P)
+_split_ok = _lib.hyb_sink_attention_split_ok
+_split_ok.argtypes = [_I, _I]
+_split_ok.restype = _I
 _prep = _sig("hyb_delta_prepare", _P, _L, _I, _I, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P,
              _P, _P, _L, _I, _I, _I, _I, _I, _I, _P)
 _scan = _sig("hyb_delta_scan", _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P)
@@ -204,7 +209,38 @@ def _i32c(t):
     return t
 
 
-def sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens, scale, sink, gate, out):
+def decode_splits(batch: int, kv_heads: int, heads: int, max_context_len) -> int:
+    """Workgroups per (sequence, KV head group) of the split decode kernel: enough to fill the
+    256 CUs several times over, each with at least 128 keys of the longest context."""
+    groups = kv_heads * -(-(heads // kv_heads) // 4)
+    want = max(1, 2048 // max(batch * groups, 1))
+    room = max(1, (int(max_context_len) + 127) // 128) if max_context_len else 8
+    return max(1, min(16, want, room))
+
+
+def sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens, scale, sink, gate, out,
+                          max_context_len=None):
+    """Single next tokens: row b is sequence b with ``context_lens[b]`` keys.  Head sizes the
+    split-context kernel has an instance for (D in 64 / 128 / 256, E in 64 / 128) stream K / V
+    rows with coalesced 16-byte loads over several workgroups per sequence and are merged by a
+    second small kernel; other sizes go through the row kernel."""
+    B, H, D = q.shape
+    G, E = k_cache.shape[2], v_cache.shape[3]
+    es = q.element_size()
+    if (_split_ok(D, E) and q.stride(2) == 1 and q.stride(1) == D and q.data_ptr() % 16 == 0
+            and (B == 1 or (q.stride(0) * es) % 16 == 0) and k_cache.is_contiguous()
+            and v_cache.is_contiguous() and out.is_contiguous()):
+        splits = decode_splits(B, G, H, max_context_len)
+        ws = torch.empty((B * H * splits * (E + 2),), dtype=torch.float32, device=q.device)
+        if gate is not None:
+            assert gate.stride(1) == 1 and gate.dtype == q.dtype
+        _check(_split(q.data_ptr(), q.stride(0) if B > 1 else H * D, q.stride(1), k_cache.data_ptr(),
+                      v_cache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0),
+                      k_cache.shape[1], _i32c(context_lens).data_ptr(), _f32(sink).data_ptr(),
+                      _ptr(gate), gate.stride(0) if gate is not None else 0, out.data_ptr(),
+                      ws.data_ptr(), scale, B, H, G, D, E, splits, _dt(q), _stream()),
+               "sink_attention_decode")
+        return out
     return _attention_rows(q, k_cache, v_cache, block_tables, None, context_lens, 0, scale, sink,
                            gate, out)
 

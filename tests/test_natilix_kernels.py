@@ -157,6 +157,29 @@ def test_sink_attention_prefill_long_portions(dt, H, G, D, E):
     torch.testing.assert_close(og.cpu().float(), o.float(), **tol(dt))
 
 
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("H,G,D,E,maxctx", [(4, 2, 128, 128, 2000), (8, 1, 64, 64, None), (2, 2, 256, 128, 300),
+                                            (6, 2, 128, 64, 100000)])
+def test_sink_attention_decode_split_contexts(dt, H, G, D, E, maxctx):
+    """The head sizes of the split-context decode kernel: several splits, contexts shorter
+    than a split, rows without a sequence, q rows strided as inside a projection output."""
+    torch.manual_seed(7)
+    bs = 16
+    lens = [1, 1500, 0, 17, 257, 640]
+    kc, vc, tables = _paged(lens, bs, G, D, E, dt)
+    kc = 0.3 * kc
+    B = len(lens)
+    proj = torch.randn(B, H * D + 24).to(dt)
+    gate, sink = torch.randn(B, H).to(dt), torch.randn(H)
+    cl = torch.tensor(lens, dtype=torch.int32)
+    o = ref.sink_attention_decode(proj[:, :H * D].view(B, H, D), kc, vc, tables, cl, D ** -0.5, sink, gate,
+                                  torch.zeros(B, H, E, dtype=dt))
+    pg = proj.cuda()
+    og = hk.sink_attention_decode(pg[:, :H * D].view(B, H, D), *dev(kc, vc, tables, cl), D ** -0.5,
+                                  sink.cuda(), gate.cuda(), torch.zeros(B, H, E, dtype=dt).cuda(), maxctx)
+    torch.testing.assert_close(og.cpu().float(), o.float(), **tol(dt))
+
+
 def test_sink_decides_when_scores_are_low():
     """A large sink takes nearly all of the weight: the output shrinks towards zero."""
     H, G, D, E, bs = 2, 1, 8, 4, 4
