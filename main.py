@@ -13,6 +13,7 @@ tokens), budgets are sized for one MI355X, and when no Qwen3 tokenizer is availa
 byte-level tokenizer is used instead of downloading one.
 """
 import argparse
+import os
 import sys
 from pathlib import Path
 
@@ -44,7 +45,8 @@ def main():
     ap.add_argument("--device", default="auto")
     ap.add_argument("--tiny", action="store_true", help="tiny model + short generation (CPU check)")
     ap.add_argument("--max-tokens", type=int, default=256)
-    ap.add_argument("--checkpoint", default=None, help="HF Qwen3 safetensors directory")
+    ap.add_argument("--checkpoint", default=None,
+                    help="checkpoint folder (config.json + safetensors) of any supported family")
     ap.add_argument("--show", type=int, default=0, help="print the first N completions")
     a = ap.parse_args()
     cfg = dict(config, model_preset=a.model, world_size=a.world_size, device=a.device,
@@ -52,6 +54,12 @@ def main():
     if a.checkpoint:
         cfg["checkpoint_path"] = a.checkpoint
         cfg["model_name_or_path"] = a.checkpoint
+        if os.path.exists(os.path.join(a.checkpoint, "config.json")):
+            # the folder says which family it is (Qwen3 / Qwen2.5 / Llama / Mistral / Natilix)
+            from minivllm_amd.models.registry import config_from_path
+            cfg.pop("model_preset")
+            cfg["model"] = config_from_path(a.checkpoint)
+            cfg["max_model_length"] = min(cfg["max_model_length"], cfg["model"].max_position)
     if a.tiny:
         cfg.update(model_preset="qwen3-tiny", max_position=2048, max_model_length=1024,
                    max_num_batched_tokens=2048,

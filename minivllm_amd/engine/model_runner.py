@@ -558,8 +558,12 @@ class ModelRunner:
         """One prefill of the largest batch the scheduler can emit, without a KV cache, so
         that peak activation memory is known before the cache is sized
         (reference: model_runner.py:129-137)."""
-        if not self.on_gpu or self.hybrid:
-            return               # (hybrid models size their caches from a fixed head-room)
+        if not self.on_gpu:
+            return
+        if self.hybrid:          # these size their caches from a computed head-room instead
+            torch.cuda.empty_cache()
+            torch.cuda.reset_peak_memory_stats()      # (an earlier engine's peak is not ours)
+            return
         cfg = self.cfg
         torch.cuda.empty_cache()
         torch.cuda.reset_peak_memory_stats()
