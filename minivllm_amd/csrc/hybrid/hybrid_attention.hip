@@ -182,7 +182,13 @@ sink_attention_rows_kernel(const T* __restrict__ q, long q_row, long q_head,
 // head sizes rounded up to the template's register arrays (padding columns of K are zeroed).
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 
-template <typename T, int DP, int EP>
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+
+// QK16 (bfloat16 caches only): the score products run as v_mfma_f32_32x32x16_bf16 on the raw
+// 16-bit K tile and q rows - the operands ARE bfloat16 values, so the products are exact and the
+// fp32 accumulation only differs in order from the fp32 instruction; the score scale is applied
+// to the fp32 result.  Weights and weighted sums stay on the fp32 instruction.
+template <typename T, int DP, int EP, bool QK16>
 __global__ void __launch_bounds__(256)
 sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
                             const T* __restrict__ k_cache, const T* __restrict__ v_cache,
@@ -192,8 +198,10 @@ sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
                             long gate_row, T* __restrict__ out, float scale, int H, int G, int D,
                             int E, int seq0, int vec_k, int vec_v) {
     extern __shared__ float sm[];
-    constexpr int KS = DP + 1;
+    constexpr int KS = QK16 ? (DP + 8) / 2 : DP + 1;      // floats per K row of the LDS image
+    constexpr int KSB = DP + 8;                             // (QK16) 16-bit elements per K row
     float* Ks = sm;
+    uint16_t* Kb = reinterpret_cast<uint16_t*>(sm);
     float* Vs = sm + 32 * KS;
     const int b = blockIdx.x + seq0, tile = blockIdx.y, h = blockIdx.z;
     const int row0 = cu_q[b], qlen = cu_q[b + 1] - row0;
@@ -206,18 +214,33 @@ sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
     const bool qok = qi < qlen;
     const int qpos = start + qi;
 
-    float qreg[DP / 2];
+    float qreg[QK16 ? 1 : DP / 2];
+    bf16x8 qv[QK16 ? DP / 16 : 1];
     {
         const T* qp = q + (long)(row0 + (qok ? qi : 0)) * q_row + (long)h * q_head;
+        if constexpr (QK16) {
 #pragma unroll
-        for (int s = 0; s < DP / 2; ++s) {
-            const int d = 2 * s + half;
-            qreg[s] = (qok && d < D) ? ld(qp + d) * scale : 0.f;
+            for (int s = 0; s < DP / 16; ++s) {
+                const int d = 16 * s + 8 * half;
+                uint4 raw = make_uint4(0, 0, 0, 0);
+                if (qok && d < D) raw = *reinterpret_cast<const uint4*>(qp + d);
+                qv[s] = __builtin_bit_cast(bf16x8, raw);
+            }
+            for (int i = tid; i < 32 * (KSB - D); i += 256) {   // padding columns of K stay zero
+                const int key = i / (KSB - D), c = D + i - key * (KSB - D);
+                Kb[key * KSB + c] = 0;
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < DP / 2; ++s) {
+                const int d = 2 * s + half;
+                qreg[s] = (qok && d < D) ? ld(qp + d) * scale : 0.f;
+            }
+            for (int i = tid; i < 32 * (KS - D); i += 256) {      // padding columns of K stay zero
+                const int key = i / (KS - D), c = D + i - key * (KS - D);
+                Ks[key * KS + c] = 0.f;
+            }
         }
-    }
-    for (int i = tid; i < 32 * (KS - D); i += 256) {          // padding columns of K stay zero
-        const int key = i / (KS - D), c = D + i - key * (KS - D);
-        Ks[key * KS + c] = 0.f;
     }
     float m = sink[h], lsum = 1.f;
     f32x16 oacc[EP / 32];
@@ -232,7 +255,18 @@ sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
 
     for (int k0 = 0; k0 < wg_ctx; k0 += 32) {
         // ---- K and V tile into LDS
-        if (vec_k) {
+        if constexpr (QK16) {
+            const int D8 = D >> 3;
+            for (int i = tid; i < 32 * D8; i += 256) {
+                const int key = i / D8, c = (i - key * D8) << 3, j = k0 + key;
+                uint4 raw = make_uint4(0, 0, 0, 0);
+                if (j < wg_ctx) {
+                    const long slot = (long)table[j / block_size] * block_size + j % block_size;
+                    raw = *reinterpret_cast<const uint4*>(k_cache + (slot * G + g) * (long)D + c);
+                }
+                *reinterpret_cast<uint4*>(Kb + key * KSB + c) = raw;
+            }
+        } else if (vec_k) {
             const int D4 = D >> 2;
             for (int i = tid; i < 32 * D4; i += 256) {
                 const int key = i / D4, c = (i - key * D4) << 2, j = k0 + key;
@@ -283,10 +317,21 @@ sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
             f32x16 sacc;
 #pragma unroll
             for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
-            const float* ka = Ks + l32 * KS + half;
+            if constexpr (QK16) {
+                const uint16_t* ka = Kb + l32 * KSB + 8 * half;
 #pragma unroll
-            for (int s = 0; s < DP / 2; ++s)
-                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[2 * s], qreg[s], sacc, 0, 0, 0);
+                for (int s = 0; s < DP / 16; ++s) {
+                    const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(ka + 16 * s));
+                    sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qv[s], sacc, 0, 0, 0);
+                }
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sacc[r] *= scale;
+            } else {
+                const float* ka = Ks + l32 * KS + half;
+#pragma unroll
+                for (int s = 0; s < DP / 2; ++s)
+                    sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[2 * s], qreg[s], sacc, 0, 0, 0);
+            }
             float mt = -INFINITY;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
@@ -342,14 +387,25 @@ static int launch_tiles(const void* q, long q_row, long q_head, const void* k_ca
                         const void* gate, long gate_row, void* out, float scale, int nseq,
                         int seq0, int max_q, int H, int G, int D, int E, int esize,
                         hipStream_t s) {
-    const size_t lds = (32 * (DP + 1) + 32 * EP) * sizeof(float);
     const int vec_k = (D % 4 == 0) && ((size_t)k_cache % 16 == 0);
     const int vec_v = (E % 4 == 0) && ((size_t)v_cache % 16 == 0);
-    hipLaunchKernelGGL((sink_attention_tiles_kernel<T, DP, EP>), dim3(nseq, (max_q + 127) / 128, H),
-                       dim3(256), lds, s, (const T*)q, q_row, q_head, (const T*)k_cache,
-                       (const T*)v_cache, (const int*)block_tables, max_blocks, block_size,
-                       (const int*)cu_q, (const int*)positions, (const float*)sink,
-                       (const T*)gate, gate_row, (T*)out, scale, H, G, D, E, seq0, vec_k, vec_v);
+    const dim3 grid(nseq, (max_q + 127) / 128, H);
+#define TILES_LAUNCH(QK16, lds)                                                                   \
+    hipLaunchKernelGGL((sink_attention_tiles_kernel<T, DP, EP, QK16>), grid, dim3(256), lds, s,   \
+                       (const T*)q, q_row, q_head, (const T*)k_cache, (const T*)v_cache,          \
+                       (const int*)block_tables, max_blocks, block_size, (const int*)cu_q,        \
+                       (const int*)positions, (const float*)sink, (const T*)gate, gate_row,       \
+                       (T*)out, scale, H, G, D, E, seq0, vec_k, vec_v)
+    if constexpr (sizeof(T) == 2) {
+        // 16-bit caches: score products on the bf16 instruction when rows are 16-byte addressable
+        if (D % 16 == 0 && (size_t)k_cache % 16 == 0 && (size_t)q % 16 == 0 && q_row % 8 == 0 &&
+            q_head % 8 == 0) {
+            TILES_LAUNCH(true, (32 * ((DP + 8) / 2) + 32 * EP) * sizeof(float));
+            return HYB_LAUNCH_OK();
+        }
+    }
+    TILES_LAUNCH(false, (32 * (DP + 1) + 32 * EP) * sizeof(float));
+#undef TILES_LAUNCH
     return HYB_LAUNCH_OK();
 }
 

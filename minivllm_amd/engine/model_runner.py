@@ -733,7 +733,7 @@ class ModelRunner:
                       block_tables=tables)
         if num_decode:
             arrays["context_lens"] = ends[:num_decode].astype(np.int32)
-        if self.on_gpu:
+        if self.on_gpu and not self.hybrid:
             # the attention kernel's work list: one entry per pair of query tiles of a prompt
             # (sequence numbers count from the first prompt)
             from minivllm_amd.ops import hip
