@@ -18,21 +18,6 @@ constexpr int TILE = 256;
 constexpr int RC = 4;       // query heads per workgroup
 constexpr int NACC = 4;     // output columns per thread: RC * E <= NACC * 256
 
-template <typename T> struct Vec4;
-template <> struct Vec4<float> {
-    static __device__ __forceinline__ void load(const float* p, float* o) {
-        const float4 v = *reinterpret_cast<const float4*>(p);
-        o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
-    }
-};
-template <> struct Vec4<bf16_t> {
-    static __device__ __forceinline__ void load(const bf16_t* p, float* o) {
-        const uint2 v = *reinterpret_cast<const uint2*>(p);
-        o[0] = __uint_as_float(v.x << 16); o[1] = __uint_as_float(v.x & 0xffff0000u);
-        o[2] = __uint_as_float(v.y << 16); o[3] = __uint_as_float(v.y & 0xffff0000u);
-    }
-};
-
 template <typename T>
 __global__ void __launch_bounds__(TILE)
 sink_attention_rows_kernel(const T* __restrict__ q, long q_row, long q_head,
@@ -417,11 +402,6 @@ static int launch_tiles(const void* q, long q_row, long q_head, const void* k_ca
 // the groups' partials meet in LDS, the workgroups' (one per context split) in a workspace that
 // `sink_attention_merge_kernel` folds together with the sink term and the gate.
 // EPL / VPL: elements of a K / V row per lane (D = 16 EPL, E = 16 VPL).
-template <typename T, int N> __device__ __forceinline__ void load_run(const T* p, float* o) {
-#pragma unroll
-    for (int i = 0; i < N; i += 4) Vec4<T>::load(p + i, o + i);
-}
-
 template <typename T, int EPL, int VPL>
 __global__ void __launch_bounds__(256)
 sink_attention_split_kernel(const T* __restrict__ q, long q_row, long q_head,
@@ -458,32 +438,42 @@ sink_attention_split_kernel(const T* __restrict__ q, long q_row, long q_head,
 #pragma unroll
         for (int i = 0; i < VPL; ++i) acc[r][i] = 0.f;
     }
-    for (int j = k_begin + kg; j < k_end; j += 16) {
+    // two keys per trip: both rows' loads are in flight before the first one is used
+    for (int j = k_begin + kg; j < k_end; j += 32) {
+        const int j2 = j + 16;
+        const bool two = j2 < k_end;
         const long slot = (long)table[j / block_size] * block_size + j % block_size;
-        float kf[EPL], vf[VPL];
-        load_run<T, EPL>(k_cache + (slot * G + g) * (long)D + lane16 * EPL, kf);
-        load_run<T, VPL>(v_cache + (slot * G + g) * (long)E + lane16 * VPL, vf);
+        const long slot2 = two ? (long)table[j2 / block_size] * block_size + j2 % block_size : slot;
+        float kf[2][EPL], vf[2][VPL];
+        load_run<T, EPL>(k_cache + (slot * G + g) * (long)D + lane16 * EPL, kf[0]);
+        load_run<T, EPL>(k_cache + (slot2 * G + g) * (long)D + lane16 * EPL, kf[1]);
+        load_run<T, VPL>(v_cache + (slot * G + g) * (long)E + lane16 * VPL, vf[0]);
+        load_run<T, VPL>(v_cache + (slot2 * G + g) * (long)E + lane16 * VPL, vf[1]);
 #pragma unroll
-        for (int r = 0; r < RC; ++r) {
-            if (r >= nr) continue;
-            float d = 0.f;
+        for (int x = 0; x < 2; ++x) {
+            if (x == 1 && !two) break;
 #pragma unroll
-            for (int i = 0; i < EPL; ++i) d += kf[i] * qf[r][i];
-            d += __shfl_xor(d, 1, kWave);
-            d += __shfl_xor(d, 2, kWave);
-            d += __shfl_xor(d, 4, kWave);
-            d += __shfl_xor(d, 8, kWave);
-            if (d > m[r]) {                        // the running maximum moves: rescale (rare)
-                const float a = expf(m[r] - d);
-                l[r] *= a;
+            for (int r = 0; r < RC; ++r) {
+                if (r >= nr) continue;
+                float d = 0.f;
 #pragma unroll
-                for (int i = 0; i < VPL; ++i) acc[r][i] *= a;
-                m[r] = d;
+                for (int i = 0; i < EPL; ++i) d += kf[x][i] * qf[r][i];
+                d += __shfl_xor(d, 1, kWave);
+                d += __shfl_xor(d, 2, kWave);
+                d += __shfl_xor(d, 4, kWave);
+                d += __shfl_xor(d, 8, kWave);
+                if (d > m[r]) {                    // the running maximum moves: rescale (rare)
+                    const float a = expf(m[r] - d);
+                    l[r] *= a;
+#pragma unroll
+                    for (int i = 0; i < VPL; ++i) acc[r][i] *= a;
+                    m[r] = d;
+                }
+                const float p = expf(d - m[r]);
+                l[r] += p;
+#pragma unroll
+                for (int i = 0; i < VPL; ++i) acc[r][i] += p * vf[x][i];
             }
-            const float p = expf(d - m[r]);
-            l[r] += p;
-#pragma unroll
-            for (int i = 0; i < VPL; ++i) acc[r][i] += p * vf[i];
         }
     }
     // the 16 groups' partials -> LDS -> one partial per (head, split)

@@ -61,6 +61,27 @@ __device__ __forceinline__ float siluf_(float z) { return z / (1.f + expf(-z)); 
 __device__ __forceinline__ float softplusf_(float z) { return z > 20.f ? z : log1pf(expf(z)); }
 __device__ __forceinline__ float gelu_erf(float z) { return 0.5f * z * (1.f + erff(z * 0.70710678118654752f)); }
 
+// four (Vec4) or N (load_run, N % 4 == 0) consecutive elements widened to fp32; the address must
+// be aligned to the run of four (8 bytes for bfloat16, 16 for float)
+template <typename T> struct Vec4;
+template <> struct Vec4<float> {
+    static __device__ __forceinline__ void load(const float* p, float* o) {
+        const float4 v = *reinterpret_cast<const float4*>(p);
+        o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+    }
+};
+template <> struct Vec4<bf16_t> {
+    static __device__ __forceinline__ void load(const bf16_t* p, float* o) {
+        const uint2 v = *reinterpret_cast<const uint2*>(p);
+        o[0] = __uint_as_float(v.x << 16); o[1] = __uint_as_float(v.x & 0xffff0000u);
+        o[2] = __uint_as_float(v.y << 16); o[3] = __uint_as_float(v.y & 0xffff0000u);
+    }
+};
+template <typename T, int N> __device__ __forceinline__ void load_run(const T* p, float* o) {
+#pragma unroll
+    for (int i = 0; i < N; i += 4) Vec4<T>::load(p + i, o + i);
+}
+
 #define HYB_DISPATCH(dt, ...)                                         \
     do {                                                              \
         if ((dt) == 0) { using T = hyb::bf16_t; __VA_ARGS__; }        \

@@ -15,9 +15,9 @@ constexpr int MAX_TAPS = 32;
 // One workgroup per token row.  proj row = [q (G*D) | k (G*D) | v (H*E) | gate | b (H) | a (H)];
 // the three convolved blocks are contiguous at the row's start (C = 2GD + HE channels).
 // conv_w [C, taps] (q, k, v rows stacked), conv_state [slots, taps-1, C].
-template <typename T>
+template <typename T, int TAPS>
 __global__ void delta_prepare_kernel(const T* __restrict__ proj, long row_stride, int b_off,
-                                     int a_off, const float* __restrict__ conv_w, int taps,
+                                     int a_off, const float* __restrict__ conv_w, int taps_rt,
                                      const float* __restrict__ a_log,
                                      const float* __restrict__ dt_bias,
                                      const float* __restrict__ conv_state,
@@ -25,8 +25,10 @@ __global__ void delta_prepare_kernel(const T* __restrict__ proj, long row_stride
                                      const int* __restrict__ slots, const int* __restrict__ row_seq,
                                      float* __restrict__ qn, float* __restrict__ kn,
                                      float* __restrict__ vv, float* __restrict__ beta,
-                                     float* __restrict__ decay, int H, int G, int D, int E) {
+                                     float* __restrict__ decay, int H, int G, int D, int E,
+                                     int vec8) {
     extern __shared__ float y[];                     // [2GD] convolved + silu q, k
+    const int taps = TAPS ? TAPS : taps_rt;          // TAPS > 0: known at compile time (unrolled)
     const long t = blockIdx.x;
     const int b = row_seq ? row_seq[t] : (int)t;
     if (b < 0) return;
@@ -37,6 +39,39 @@ __global__ void delta_prepare_kernel(const T* __restrict__ proj, long row_stride
     const bool has_past = positions[first] > 0;
     const int C = 2 * G * D + H * E, GD = G * D;
     const float* tail = conv_state + (long)slot * (taps - 1) * C;
+    if (TAPS > 0 && vec8) {
+        // eight channels per thread and step, every load of the step issued before its first use:
+        // one 16-byte (bf16) load per tap and the channels' taps as whole rows of the tap table
+        constexpr int NT = TAPS ? TAPS : 1;
+        for (int c = threadIdx.x * 8; c < C; c += blockDim.x * 8) {
+            float x[NT][8], w[8][NT];
+#pragma unroll
+            for (int j = 0; j < NT; ++j) {
+                const int back = NT - 1 - j;
+                if (i - back >= 0) load_run<T, 8>(proj + (t - back) * row_stride + c, x[j]);
+                else if (has_past) load_run<float, 8>(tail + (long)(NT - 1 + i - back) * C + c, x[j]);
+                else {
+#pragma unroll
+                    for (int z = 0; z < 8; ++z) x[j][z] = 0.f;
+                }
+            }
+#pragma unroll
+            for (int z = 0; z < 8; ++z)
+#pragma unroll
+                for (int j = 0; j < NT; ++j) w[z][j] = conv_w[(long)(c + z) * NT + j];
+            float acc[8];
+#pragma unroll
+            for (int z = 0; z < 8; ++z) {
+                float a = 0.f;
+#pragma unroll
+                for (int j = 0; j < NT; ++j) a += x[j][z] * w[z][j];
+                acc[z] = siluf_(a);
+            }
+            float* dst = (c < 2 * GD) ? y + c : vv + t * (long)(H * E) + (c - 2 * GD);
+            *reinterpret_cast<float4*>(dst) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+            *reinterpret_cast<float4*>(dst + 4) = make_float4(acc[4], acc[5], acc[6], acc[7]);
+        }
+    } else
     for (int c = threadIdx.x; c < C; c += blockDim.x) {
         float acc = 0.f;
         for (int j = 0; j < taps; ++j) {             // tap j reads the input `taps-1-j` tokens back
@@ -188,32 +223,36 @@ delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
         const float* buf = sm + (ch & 1) * BUF;
         if (ch + 1 < nchunks) fetch(ch + 1, reg);
         const int nt = min(CT, n - ch * CT);
+#pragma unroll 2
         for (int tok = 0; tok < nt; ++tok) {
             const float4* kp = reinterpret_cast<const float4*>(buf + (tok * 4 + r) * RS);
             const float4* qp = reinterpret_cast<const float4*>(buf + KQ + (tok * 4 + r) * RS);
             const float ve = buf[2 * KQ + tok * 64 + c];
             const float bt = buf[2 * KQ + CT * 64 + tok], gd = buf[2 * KQ + CT * 64 + CT + tok];
-            float kc[NR];
-            float dot = 0.f;
+            float4 k4[NR / 4], q4[NR / 4];
+#pragma unroll
+            for (int i = 0; i < NR / 4; ++i) { k4[i] = kp[i]; q4[i] = qp[i]; }
+            // four partial sums each: a single chain of NR dependent FMAs would be what a step
+            // waits for (one wave per SIMD: nobody else fills the gaps)
+            float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
 #pragma unroll
             for (int i = 0; i < NR / 4; ++i) {
-                const float4 k4 = kp[i];
-                kc[4 * i] = k4.x; kc[4 * i + 1] = k4.y; kc[4 * i + 2] = k4.z; kc[4 * i + 3] = k4.w;
+                d0 += S[4 * i] * k4[i].x; d1 += S[4 * i + 1] * k4[i].y;
+                d2 += S[4 * i + 2] * k4[i].z; d3 += S[4 * i + 3] * k4[i].w;
             }
-#pragma unroll
-            for (int i = 0; i < NR; ++i) dot += S[i] * kc[i];
+            float dot = (d0 + d1) + (d2 + d3);
             dot += __shfl_xor(dot, 1, kWave);
             dot += __shfl_xor(dot, 2, kWave);
             const float u = bt * (ve - gd * dot);
-            float out = 0.f;
+            float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
             for (int i = 0; i < NR / 4; ++i) {
-                const float4 q4 = qp[i];
-                S[4 * i] = gd * S[4 * i] + kc[4 * i] * u;             out += S[4 * i] * q4.x;
-                S[4 * i + 1] = gd * S[4 * i + 1] + kc[4 * i + 1] * u; out += S[4 * i + 1] * q4.y;
-                S[4 * i + 2] = gd * S[4 * i + 2] + kc[4 * i + 2] * u; out += S[4 * i + 2] * q4.z;
-                S[4 * i + 3] = gd * S[4 * i + 3] + kc[4 * i + 3] * u; out += S[4 * i + 3] * q4.w;
+                S[4 * i] = gd * S[4 * i] + k4[i].x * u;         o0 += S[4 * i] * q4[i].x;
+                S[4 * i + 1] = gd * S[4 * i + 1] + k4[i].y * u; o1 += S[4 * i + 1] * q4[i].y;
+                S[4 * i + 2] = gd * S[4 * i + 2] + k4[i].z * u; o2 += S[4 * i + 2] * q4[i].z;
+                S[4 * i + 3] = gd * S[4 * i + 3] + k4[i].w * u; o3 += S[4 * i + 3] * q4[i].w;
             }
+            float out = (o0 + o1) + (o2 + o3);
             out += __shfl_xor(out, 1, kWave);
             out += __shfl_xor(out, 2, kWave);
             if (col && r == 0) o[((first + ch * CT + tok) * H + h) * (long)E + e] = out;
@@ -252,14 +291,22 @@ int hyb_delta_prepare(const void* proj, long row_stride, int b_off, int a_off, c
     const int C = 2 * G * D + H * E;
     const size_t lds = 2 * (size_t)G * D * sizeof(float);
     if (lds > 64 * 1024) return 1;
-    HYB_DISPATCH(dt, hipLaunchKernelGGL(delta_prepare_kernel<T>, dim3(T_), dim3(C >= 2048 && T_ <= 1024 ? 1024 : 256),
-                                        lds, s,
-                                        (const T*)proj, row_stride, b_off, a_off,
-                                        (const float*)conv_w, taps, (const float*)a_log,
-                                        (const float*)dt_bias, (const float*)conv_state,
-                                        (const int*)cu_q, (const int*)positions, (const int*)slots,
-                                        (const int*)row_seq, (float*)qn, (float*)kn, (float*)vv,
-                                        (float*)beta, (float*)decay, H, G, D, E));
+    const int vec8 = (G * D) % 8 == 0 && (H * E) % 8 == 0 && row_stride % 8 == 0 &&
+                     (size_t)proj % 16 == 0 && (size_t)conv_state % 16 == 0 && (size_t)vv % 16 == 0;
+#define PREP(TAPS)                                                                                 \
+    HYB_DISPATCH(dt, hipLaunchKernelGGL((delta_prepare_kernel<T, TAPS>), dim3(T_),                 \
+                                        dim3(C >= 2048 && T_ <= 1024 ? 1024 : 256), lds, s,        \
+                                        (const T*)proj, row_stride, b_off, a_off,                  \
+                                        (const float*)conv_w, taps, (const float*)a_log,           \
+                                        (const float*)dt_bias, (const float*)conv_state,           \
+                                        (const int*)cu_q, (const int*)positions, (const int*)slots,\
+                                        (const int*)row_seq, (float*)qn, (float*)kn, (float*)vv,   \
+                                        (float*)beta, (float*)decay, H, G, D, E, vec8))
+    if (taps == 4) PREP(4);
+    else if (taps == 3) PREP(3);
+    else if (taps == 2) PREP(2);
+    else PREP(0);
+#undef PREP
     if (hipGetLastError() != hipSuccess) return 2;
     if (taps > 1) {
         HYB_DISPATCH(dt, hipLaunchKernelGGL(delta_conv_tail_kernel<T>, dim3(B, (C + 255) / 256),
