@@ -1027,8 +1027,10 @@ class ModelRunner:
     def _can_prelaunch(self, b: Batch) -> bool:
         if b.is_prefill or not self.cfg.decode_prelaunch or "top_k" in b.arrays:
             return False
-        if self.needs_aux_rows:
-            return False     # the next step's embedding rows depend on the token sampled now
+        if self.hybrid:
+            # the step derived on the device carries neither state slots nor the embedding rows
+            # that depend on the token sampled now
+            return False
         if os.environ.get("MINIVLLM_NO_PRELAUNCH") == "1":
             return False
         if self.on_gpu and self._graph_bucket(b.num_seqs) is None:
