@@ -301,7 +301,7 @@ def hybrid_models(size: str, vocab: int = 32768, experts: int = 4, top: int = 2)
     hybrid = NatilixConfig.from_dict({"architecture": "Natilix", "vocab": vocab, "width": W,
                                       "norm": {"eps": 1e-6}, "layers": layers,
                                       "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31,
-                                                               "mul_cur": 17}},
+                                                               "mul_cur": 13}},
                                       "max_position": 8192}, name=f"natilix-{size}")
     dense = ModelConfig(vocab_size=vocab, hidden_size=W, num_heads=H, num_kv_heads=G, head_dim=D,
                         intermediate_size=inter, num_layers=L, max_position=8192,

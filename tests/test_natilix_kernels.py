@@ -85,7 +85,7 @@ def _paged(T_lens, bs, G, D, E, dt):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
-@pytest.mark.parametrize("H,G,D,E", [(4, 2, 64, 32), (5, 1, 20, 12), (8, 8, 16, 40), (12, 2, 32, 8)])
+@pytest.mark.parametrize("H,G,D,E", [(4, 2, 64, 48), (5, 1, 20, 12), (8, 8, 16, 40), (12, 2, 32, 8)])
 def test_sink_attention_decode_and_step(dt, H, G, D, E):
     torch.manual_seed(2)
     bs = 16
@@ -195,7 +195,7 @@ def test_sink_decides_when_scores_are_low():
 
 
 @pytest.mark.parametrize("dt", DTYPES)
-@pytest.mark.parametrize("H,G,D,E,taps", [(4, 2, 32, 32, 4), (3, 1, 20, 12, 2), (4, 4, 70, 40, 1),
+@pytest.mark.parametrize("H,G,D,E,taps", [(4, 2, 32, 48, 4), (3, 1, 20, 12, 2), (4, 4, 70, 40, 1),
                                           (2, 1, 128, 96, 5)])
 def test_delta_prepare_and_scan(dt, H, G, D, E, taps):
     torch.manual_seed(3)
@@ -249,7 +249,7 @@ def test_gated_head_norm_route_and_gelu(dt):
     o, w, gate = torch.randn(T, H, E), 1 + 0.1 * torch.randn(E), torch.randn(T, H * E).to(dt)
     torch.testing.assert_close(hk.gated_head_norm(*dev(o, w, gate), 1e-5, dt).cpu().float(),
                                ref.gated_head_norm(o, w, gate, 1e-5, dt).float(), **tol(dt))
-    for NE, top, groups, keep, W in ((8, 4, 2, 1, 64), (12, 3, 4, 2, 100), (6, 2, 1, 1, 33), (16, 1, 16, 3, 40)):
+    for NE, top, groups, keep, W in ((8, 3, 2, 1, 64), (12, 3, 4, 2, 100), (6, 2, 1, 1, 33), (16, 1, 16, 3, 40)):
         h, wr = torch.randn(T, W).to(dt), torch.randn(NE, W)
         d = ref.grouped_route(h, wr, top, groups, keep)
         dg = hk.grouped_route(h.cuda(), wr.cuda(), top, groups, keep).cpu()
