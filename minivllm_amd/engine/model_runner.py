@@ -904,7 +904,10 @@ class ModelRunner:
         self.step_counter += 1
         batch.step = self.step_counter
         with torch.inference_mode(), trace_range("score_step"):
-            self.execute(batch)
+            if is_prefill:
+                self.execute(batch, pg_key=None)     # (captured prefill steps end in the sampler)
+            else:
+                self.execute(batch)
             logits = self._last_step_logits[:len(owner), :V].float().cpu()
         self._last_tokens = None
         self._decode_prev = None

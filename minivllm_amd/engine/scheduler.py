@@ -446,6 +446,9 @@ class Scheduler:
                     raise RuntimeError("no room to admit a sequence of the given step")
                 self.waiting.remove(seq)
                 self._allocate(seq)
+                # a given portion is computed in full, also where the prefix cache knows its
+                # first blocks (rewriting them stores the same values)
+                seq.num_cached_tokens = 0
                 seq.status = SequenceStatus.RUNNING
                 self.running.append(seq)
             elif seq.status != SequenceStatus.RUNNING:
