@@ -1,9 +1,12 @@
 // Causal attention over a paged cache with a sink term in the softmax denominator, separate key
 // and value head sizes, grouped query heads and an optional sigmoid gate per head.  fp32 scores,
-// weights and accumulation for bfloat16 and float caches alike.
+// weights and accumulation for bfloat16 and float caches alike.  Three kernels:
+//   sink_attention_tiles  - prompt portions on the matrix cores (below, second)
+//   sink_attention_split  - decode rows at serving head sizes, context split over workgroups (third)
+//   sink_attention_rows   - any head sizes, row by row: the reference form of the other two (first)
 //
-// One workgroup (256 threads) per (query row, group of up to RC query heads that share a KV
-// head).  The keys of the row's context are walked in tiles of 256: a thread scores one key of
+// sink_attention_rows: one workgroup (256 threads) per (query row, group of up to RC query heads
+// that share a KV head).  The keys of the row's context are walked in tiles of 256: a thread scores one key of
 // the tile against the RC heads (key read once), the tile's maximum and sum update the running
 // softmax, then the threads switch roles and each owns output columns (head, e) whose weighted
 // value sum it extends over the tile's keys (value rows read coalesced).  The running maximum
