@@ -219,3 +219,24 @@ def test_greedy_generation_through_the_scheduler(tmp_path, device, dtype):
             assert int(lg.argmax()) == t
             lg = orc.feed([t])[-1]
     eng.exit()
+
+
+@pytest.mark.parametrize("device,dtype", CASES[:2])
+def test_generation_survives_preemption_and_mixed_steps(tmp_path, device, dtype):
+    """A KV pool too small for all requests at once (sequences are preempted and prefetched
+    again from position 0: their state slot and blocks have been used by others meanwhile) and
+    running sequences riding along with prefill steps: greedy tokens still equal the oracle's."""
+    c, w = fx.default_config(), fx.weights(fx.default_config(), 19)
+    prompts = [tokens(n, c["vocab"], 60 + n) for n in (21, 17, 9, 30)]
+    eng = make_engine(tmp_path, c, w, device, dtype, score=False, seqs=3, blocks=11, block_size=8,
+                      max_num_batched_tokens=24, enable_mixed_batches=True)
+    out = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=14, ignore_eos=True))
+    assert eng.scheduler.num_preemptions > 0 and eng.scheduler.num_mixed_steps > 0
+    for p, gen in zip(prompts, out["token_ids"]):
+        orc = Oracle(c, w)
+        lg = orc.feed(p)[-1]
+        for t in gen:
+            assert int(lg.argmax()) == t
+            lg = orc.feed([t])[-1]
+    assert eng.scheduler.state_pool.num_free == 3
+    eng.exit()
