@@ -517,7 +517,8 @@ class ModelRunner:
             attn.k_cache = attn.v_cache = None
         if self.hybrid:
             for d in self.model.state_layers():
-                d.state = d.conv_state = None
+                for attr, _ in d.state_spec():
+                    setattr(d, attr, None)
         self.kv_cache = None
         self.model = None
         self._dec_dev = self._pre_dev = None
@@ -647,9 +648,8 @@ class ModelRunner:
             attn.block_size = self.block_size
 
     def _state_bytes(self) -> int:
-        return sum(self.num_state_slots * 4 * (d.num_heads * d.head_dim * d.v_head_dim
-                                               + max(d.taps - 1, 0) * d.conv_channels)
-                   for d in self.model.state_layers())
+        return sum(self.num_state_slots * 4 * int(np.prod(shape, dtype=np.int64))
+                   for d in self.model.state_layers() for _, shape in d.state_spec())
 
     def _widest_row_bytes(self) -> int:
         widest = max([p.shape[0] for p in self.model.parameters() if p.dim() == 2] + [1])
@@ -658,7 +658,8 @@ class ModelRunner:
     def _allocate_hybrid_caches(self) -> None:
         """One K and one V allocation per attention layer (their head sizes may differ from
         layer to layer and between K and V), logical [block, token, kv head, d]; per recurrent
-        layer a fp32 state row and a convolution-tail row for every state slot."""
+        layer one fp32 row per state slot of whatever the layer's ``state_spec`` lists (matrix
+        state, normaliser, running maximum, convolution tail, ...)."""
         n, bs = self.num_kv_blocks, self.block_size
         self.kv_cache = []
         for a in self.model.attention_layers():
@@ -666,11 +667,9 @@ class ModelRunner:
             a.v_cache = torch.zeros(n, bs, a.num_kv_heads, a.v_head_dim, dtype=self.kv_dtype, device=self.device)
             self.kv_cache.append((a.k_cache, a.v_cache))
         for d in self.model.state_layers():
-            S = self.num_state_slots
-            d.state = torch.zeros(S, d.num_heads, d.head_dim, d.v_head_dim, dtype=torch.float32,
-                                  device=self.device)
-            d.conv_state = torch.zeros(S, max(d.taps - 1, 0), d.conv_channels, dtype=torch.float32,
-                                       device=self.device)
+            for attr, shape in d.state_spec():
+                setattr(d, attr, torch.zeros((self.num_state_slots,) + tuple(shape),
+                                             dtype=torch.float32, device=self.device))
 
     # ============================================================ batch building
     def prepare_prefill(self, seqs: Seq[Sequence], num_decode: int = 0) -> Batch:

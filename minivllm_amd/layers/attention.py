@@ -165,14 +165,26 @@ class SinkAttention(nn.Module):
     ``exp(sink_h)`` per query head (no key, no value), with key and value heads of different
     sizes (K cache [blocks, block, G, D], V cache [blocks, block, G, E]) and an optional
     per-head output gate ``sigmoid(gate_h)`` applied inside the kernel.  ``scale`` is the full
-    score multiplier.  Scores, weights and the weighted sum are fp32 in every implementation."""
+    score multiplier.  Scores, weights and the weighted sum are fp32 in every implementation.
+
+    Options, each a constructor argument: ``sink=False`` - an ordinary softmax (no extra term);
+    ``window`` > 0 - a query at position i sees key j <= i only when i - j < window or
+    j < keep_first (the first tokens stay visible at their true positions); ``distance_slopes``
+    [H] - slope_h * (i - j) is taken off the score of key j."""
 
     def __init__(self, num_heads: int, num_kv_heads: int, head_dim: int, v_head_dim: int,
-                 scale: float):
+                 scale: float, sink: bool = True, window: int = 0, keep_first: int = 0,
+                 distance_slopes: Optional[torch.Tensor] = None):
         super().__init__()
         self.num_heads, self.num_kv_heads = num_heads, num_kv_heads
         self.head_dim, self.v_head_dim, self.scale = head_dim, v_head_dim, scale
-        self.sink = nn.Parameter(torch.zeros(num_heads, dtype=torch.float32), requires_grad=False)
+        self.window, self.keep_first = int(window), int(keep_first)
+        self.sink = (nn.Parameter(torch.zeros(num_heads, dtype=torch.float32), requires_grad=False)
+                     if sink else None)
+        if distance_slopes is not None:
+            self.register_buffer("slopes", distance_slopes.to(torch.float32), persistent=False)
+        else:
+            self.slopes = None
         self.k_cache: Optional[torch.Tensor] = None
         self.v_cache: Optional[torch.Tensor] = None
 
@@ -185,9 +197,10 @@ class SinkAttention(nn.Module):
         T = q.shape[0]
         out = torch.zeros((T, self.num_heads, self.v_head_dim), dtype=q.dtype, device=q.device)
         a = (self.k_cache, self.v_cache)
+        opt = dict(window=self.window, keep_first=self.keep_first, slopes=self.slopes)
         if not ctx.is_prefill:
             ops.sink_attention_decode(q, *a, ctx.block_tables, ctx.context_lens, self.scale,
-                                      self.sink, gate, out, ctx.max_context_len or None)
+                                      self.sink, gate, out, ctx.max_context_len or None, **opt)
         else:
             # prompt portions through the prefill kernel, the single next tokens that ride along
             # (the first num_decode_seqs rows and sequences) through the decode kernel
@@ -196,10 +209,10 @@ class SinkAttention(nn.Module):
                 ops.sink_attention_prefill(q, *a, ctx.cu_seqlens_q[Bd:], ctx.cu_seqlens_k[Bd:],
                                            ctx.block_tables[Bd:], self.scale, self.sink, gate, out,
                                            positions=ctx.positions, max_q=ctx.max_seqlen_q or None,
-                                           row_seq=ctx.row_seq, first_seq=Bd)
+                                           row_seq=ctx.row_seq, first_seq=Bd, **opt)
             if Bd:
                 ops.sink_attention_decode(q[:Bd], *a, ctx.block_tables[:Bd], ctx.context_lens,
                                           self.scale, self.sink,
                                           None if gate is None else gate[:Bd], out[:Bd],
-                                          ctx.max_context_len or None)
+                                          ctx.max_context_len or None, **opt)
         return out.view(T, self.num_heads * self.v_head_dim)

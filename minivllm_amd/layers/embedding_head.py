@@ -17,6 +17,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from minivllm_amd import ops
 from minivllm_amd.parallel import group as pg
 from minivllm_amd.utils.context import get_context
 
@@ -100,3 +101,20 @@ class HashedBigramEmbedding(nn.Module):
         t, p = np.asarray(tokens, np.int64), np.asarray(prev_tokens, np.int64)
         rows = (p * self.mul_prev + t * self.mul_cur) % self.buckets
         return np.where(p < 0, self.buckets, rows).astype(np.int32)
+
+
+class SinusoidalEmbedding(nn.Module):
+    """Token rows plus a fixed position vector: entry 2i is sin(p f_i), entry 2i+1 cos(p f_i),
+    f_i = base^(-2i / width).  Nothing is tabulated per position: the kernel forms the fp32 angle
+    from the position and the fp32 frequency, so any position is served.  Output fp32."""
+
+    def __init__(self, num_embeddings: int, embedding_dim: int, base: float = 10000.0):
+        super().__init__()
+        if embedding_dim % 2:
+            raise ValueError("sinusoidal positions need an even width")
+        self.weight = nn.Parameter(torch.zeros(num_embeddings, embedding_dim), requires_grad=False)
+        i = torch.arange(embedding_dim // 2, dtype=torch.float64)
+        self.register_buffer("inv_freq", (base ** (-2.0 * i / embedding_dim)).float(), persistent=False)
+
+    def forward(self, ids: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+        return ops.embed_sinusoid(ids, positions, self.weight, self.inv_freq)

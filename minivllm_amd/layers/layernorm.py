@@ -61,3 +61,20 @@ class OffsetRMSNorm(nn.Module):
 
     def forward(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
         return ops.offset_rms_norm(x, self.weight, self.eps, out_dtype or x.dtype)
+
+
+class GroupRMSNorm(nn.Module):
+    """RMS norm in groups: the vector is cut into ``groups`` equal consecutive parts, each
+    divided by its own root mean square (eps inside the root), the whole multiplied by a plain
+    fp32 weight.  ``groups`` = 1 is the ordinary RMS norm.  Applied alone (``ops.group_rms_norm``)
+    or fused with the update of a fp32 residual stream (``ops.residual_group_norm``)."""
+
+    def __init__(self, hidden_size: int, groups: int = 1, eps: float = 1e-6):
+        super().__init__()
+        if groups < 1 or hidden_size % groups:
+            raise ValueError("the norm's groups must divide the width")
+        self.eps, self.groups = eps, groups
+        self.weight = nn.Parameter(torch.ones(hidden_size, dtype=torch.float32), requires_grad=False)
+
+    def forward(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        return ops.group_rms_norm(x, self.weight, self.groups, self.eps, out_dtype or x.dtype)

@@ -37,3 +37,47 @@ class GroupedRoutedExperts(nn.Module):
         route = ops.grouped_route(h, self.router, self.top, self.groups, self.keep)
         act = ops.gelu_route_scale(F.linear(h, self.up), route, self.ff, h.dtype)
         return F.linear(act, self.down)
+
+
+class RoutedGatedExperts(nn.Module):
+    """Gated feed-forward experts down(silu(gate x) * (up x)) behind a sigmoid router, plus an
+    optional shared expert that every token uses; with ``experts`` = 0 it is a plain dense gated
+    feed-forward of size ``shared_ff``.
+
+    Router: s = sigmoid(W_r h) in fp32, the ``top`` largest scores chosen (ties to the lower
+    index) and used as weights as they are.  The weight multiplies the expert's INPUT:
+    out = sum_j expert_j(s_j h) + shared(h).
+
+    Execution: one stacked gate+up weight [2 C, W], C = experts * ff + shared_ff (all gate rows,
+    then all up rows) and one stacked down weight [W, C].  Because the two input projections are
+    linear, scaling the input by s_j is scaling their outputs, which the activation kernel does
+    (``ops.swiglu_route_scale``; exactly zero for experts a token did not choose): two dense
+    GEMMs and one elementwise kernel for routed experts, shared expert and dense layer alike,
+    no token permutation, no host synchronisation."""
+
+    def __init__(self, hidden_size: int, ff: int, experts: int, top: int, shared_ff: int = 0):
+        super().__init__()
+        if experts and not 0 < top <= experts:
+            raise ValueError("router: `top` must lie in 1 .. experts")
+        self.ff, self.experts, self.top, self.shared_ff = ff, experts, top, shared_ff
+        self.columns = experts * ff + shared_ff
+        self.router = (nn.Parameter(torch.zeros(experts, hidden_size, dtype=torch.float32),
+                                    requires_grad=False) if experts else None)
+        self.gate_up = nn.Parameter(torch.zeros(2 * self.columns, hidden_size), requires_grad=False)
+        self.down = nn.Parameter(torch.zeros(hidden_size, self.columns), requires_grad=False)
+
+    def column_range(self, expert: int):
+        """Columns of expert ``expert`` (-1: the shared one) among the stacked C."""
+        if expert < 0:
+            return self.experts * self.ff, self.columns
+        return expert * self.ff, (expert + 1) * self.ff
+
+    def forward(self, h: torch.Tensor, gu: torch.Tensor = None) -> torch.Tensor:
+        """``gu``: the stacked gate+up projection of h when the caller has computed it already
+        (as columns of a wider fused projection)."""
+        route = (ops.grouped_route(h, self.router, self.top, 1, 1, "sigmoid")
+                 if self.experts else None)
+        if gu is None:
+            gu = F.linear(h, self.gate_up)
+        act = ops.swiglu_route_scale(gu, route, self.ff, self.shared_ff, h.dtype)
+        return F.linear(act, self.down)

@@ -84,3 +84,13 @@ def _ensure_builtin() -> None:
         return NatilixForCausalLM
 
     register(["natilix"], natilix_cfg, natilix_class)
+
+    def pelenex_cfg(c, name):
+        from minivllm_amd.models.pelenex import PelenexConfig
+        return PelenexConfig.from_dict(c, name)
+
+    def pelenex_class():
+        from minivllm_amd.models.pelenex import PelenexForCausalLM
+        return PelenexForCausalLM
+
+    register(["pelenex"], pelenex_cfg, pelenex_class)

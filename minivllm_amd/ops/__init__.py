@@ -263,35 +263,45 @@ def pair_rope_mix_store(q, k, v, positions, cos_sin, rot_dims, v_first, lam, v_m
 
 
 def sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables, scale, sink, gate, out,
-                           positions=None, max_q=None, row_seq=None, first_seq=0):
+                           positions=None, max_q=None, row_seq=None, first_seq=0,
+                           window=0, keep_first=0, slopes=None):
     """``positions`` [T], ``max_q`` (longest portion, a host integer), ``row_seq`` and ``first_seq``
     (how many sequences of the step precede ``cu_q[0]``'s, i.e. what was sliced off): what the
     GPU kernels take besides (``hip_hybrid.sink_attention_prefill``); the CPU form derives
-    everything from ``cu_q`` / ``cu_k``."""
+    everything from ``cu_q`` / ``cu_k``.  ``sink`` None: no sink term.  ``window`` > 0: a query at
+    position i sees key j <= i only if i - j < window or j < keep_first.  ``slopes`` [H] fp32:
+    slope_h * (i - j) is taken off the score."""
     if _on_gpu(q):
         return _hybrid().sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables,
                                                 scale, sink, gate, out, positions=positions,
-                                                max_q=max_q, row_seq=row_seq, first_seq=first_seq)
+                                                max_q=max_q, row_seq=row_seq, first_seq=first_seq,
+                                                window=window, keep_first=keep_first, slopes=slopes)
     return torch_seqmix.sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables,
-                                               scale, sink, gate, out)
+                                               scale, sink, gate, out, window, keep_first, slopes)
 
 
 def sink_attention_step(q, k_cache, v_cache, block_tables, row_seq, positions, scale, sink, gate,
-                        out):
+                        out, window=0, keep_first=0, slopes=None):
     """GPU only: all rows of a prefill-form step in one launch (``hip_hybrid``)."""
     return _hybrid().sink_attention_step(q, k_cache, v_cache, block_tables, row_seq, positions,
-                                         scale, sink, gate, out)
+                                         scale, sink, gate, out, window=window,
+                                         keep_first=keep_first, slopes=slopes)
 
 
 def sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens, scale, sink, gate, out,
-                          max_context_len=None):
+                          max_context_len=None, window=0, keep_first=0, slopes=None):
     """``max_context_len`` (a host integer, an upper bound will do): lets the GPU form size its
     context splits without reading the lengths back."""
     if _on_gpu(q):
         return _hybrid().sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens,
-                                               scale, sink, gate, out, max_context_len)
+                                               scale, sink, gate, out, max_context_len,
+                                               window=window, keep_first=keep_first, slopes=slopes)
     return torch_seqmix.sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens,
-                                              scale, sink, gate, out)
+                                              scale, sink, gate, out, window, keep_first, slopes)
+
+
+def unit_norm_store(q, k, eps, k_cache, v_cache, slot_mapping):
+    return _seqmix(q).unit_norm_store(q, k, eps, k_cache, v_cache, slot_mapping)
 
 
 def delta_prepare(q, k, v, b, a, conv_w, a_log, dt_bias, conv_state, cu_q, positions, slots,
@@ -309,12 +319,46 @@ def delta_scan(qn, kn, vv, beta, decay, state, cu_q, positions, slots):
     return _seqmix(qn).delta_scan(qn, kn, vv, beta, decay, state, cu_q, positions, slots)
 
 
-def gated_head_norm(o, w, gate, eps, out_dtype):
-    return _seqmix(o).gated_head_norm(o, w, gate, eps, out_dtype)
+def gated_head_norm(o, w, gate, eps, out_dtype, act="silu"):
+    return _seqmix(o).gated_head_norm(o, w, gate, eps, out_dtype, act)
 
 
-def grouped_route(h, router_w, top, groups, keep):
-    return _seqmix(h).grouped_route(h, router_w, top, groups, keep)
+def grouped_route(h, router_w, top, groups, keep, score="softmax"):
+    return _seqmix(h).grouped_route(h, router_w, top, groups, keep, score)
+
+
+def swiglu_route_scale(gu, dense, ff, shared_ff, out_dtype):
+    return _seqmix(gu).swiglu_route_scale(gu, dense, ff, shared_ff, out_dtype)
+
+
+def embed_sinusoid(ids, positions, table, inv_freq):
+    return _seqmix(table).embed_sinusoid(ids, positions, table, inv_freq)
+
+
+def group_rms_norm(x, w, groups, eps, out_dtype):
+    return _seqmix(x).group_rms_norm(x, w, groups, eps, out_dtype)
+
+
+def residual_group_norm(x, ys, w_next, groups, eps, out_dtype):
+    return _seqmix(x).residual_group_norm(x, ys, w_next, groups, eps, out_dtype)
+
+
+def add_normed_mean(x, parts, eps):
+    return _seqmix(x).add_normed_mean(x, parts, eps)
+
+
+def tanh_cap_(z, cap):
+    return _seqmix(z).tanh_cap_(z, cap)
+
+
+def mlstm_scan(q, k, v, i_raw, f_raw, i_bias, f_bias, cap, state, norm_state, max_state,
+               cu_q, positions, slots):
+    return _seqmix(q).mlstm_scan(q, k, v, i_raw, f_raw, i_bias, f_bias, cap, state, norm_state,
+                                 max_state, cu_q, positions, slots)
+
+
+def gla_scan(q, k, v, a_raw, a_bias, tau, state, cu_q, positions, slots):
+    return _seqmix(q).gla_scan(q, k, v, a_raw, a_bias, tau, state, cu_q, positions, slots)
 
 
 def gelu_route_scale(up, dense, ff, out_dtype):

@@ -108,8 +108,11 @@ def pair_rope_mix_store(q, k, v, positions, cos_sin, rot_dims, v_first, lam, v_m
 
 
 # ------------------------------------------------------------------ attention with a sink
-def _sink_attend(q, k, v, scale, sink, gate, offset):
-    """q [Lq,H,D], k [Lk,G,D], v [Lk,G,E], gate [Lq,H] -> [Lq,H,E] fp32."""
+def _sink_attend(q, k, v, scale, sink, gate, offset, window=0, keep_first=0, slopes=None):
+    """q [Lq,H,D], k [Lk,G,D], v [Lk,G,E], gate [Lq,H] -> [Lq,H,E] fp32.  Query row i sits at
+    position ``offset + i`` and sees key j <= its position; with ``window`` > 0 only keys with
+    position - j < window or j < keep_first.  ``slopes`` [H]: slope_h * (position - j) is taken
+    off the score.  ``sink`` None: an ordinary softmax."""
     Lq, H, _ = q.shape
     Lk, G, _ = k.shape
     r = H // G
@@ -118,8 +121,16 @@ def _sink_attend(q, k, v, scale, sink, gate, offset):
     vf = v.float().transpose(0, 1).repeat_interleave(r, 0)
     s = torch.matmul(qf, kf.transpose(1, 2)) * scale                  # [H, Lq, Lk]
     qi = torch.arange(Lq)[:, None] + offset
-    s = s.masked_fill((torch.arange(Lk)[None, :] > qi)[None], float("-inf"))
-    s = torch.cat([s, sink.float()[:, None, None].expand(H, Lq, 1)], -1)
+    kj = torch.arange(Lk)[None, :]
+    dist = (qi - kj).float()
+    if slopes is not None:
+        s = s - slopes.float()[:, None, None] * dist[None]
+    hidden = kj > qi
+    if window:
+        hidden = hidden | ((qi - kj >= window) & (kj >= keep_first))
+    s = s.masked_fill(hidden[None], float("-inf"))
+    if sink is not None:
+        s = torch.cat([s, sink.float()[:, None, None].expand(H, Lq, 1)], -1)
     p = torch.softmax(s, -1)[..., :Lk]
     o = torch.matmul(p, vf).transpose(0, 1)                           # [Lq, H, E]
     if gate is not None:
@@ -127,7 +138,8 @@ def _sink_attend(q, k, v, scale, sink, gate, offset):
     return o
 
 
-def sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables, scale, sink, gate, out):
+def sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables, scale, sink, gate, out,
+                           window=0, keep_first=0, slopes=None):
     cq, ck = cu_q.tolist(), cu_k.tolist()
     for b in range(len(cq) - 1):
         s, e = cq[b], cq[b + 1]
@@ -137,19 +149,38 @@ def sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables, scale,
         k = _gather_paged(k_cache, block_tables[b], lk)
         v = _gather_paged(v_cache, block_tables[b], lk)
         out[s:e] = _sink_attend(q[s:e], k, v, scale, sink, None if gate is None else gate[s:e],
-                                lk - (e - s)).to(out.dtype)
+                                lk - (e - s), window, keep_first, slopes).to(out.dtype)
     return out
 
 
-def sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens, scale, sink, gate, out):
+def sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens, scale, sink, gate, out,
+                          window=0, keep_first=0, slopes=None):
     for b, L in enumerate(context_lens.tolist()):
         if L <= 0:
             continue
         k = _gather_paged(k_cache, block_tables[b], L)
         v = _gather_paged(v_cache, block_tables[b], L)
         out[b:b + 1] = _sink_attend(q[b:b + 1], k, v, scale, sink,
-                                    None if gate is None else gate[b:b + 1], L - 1).to(out.dtype)
+                                    None if gate is None else gate[b:b + 1], L - 1, window,
+                                    keep_first, slopes).to(out.dtype)
     return out
+
+
+def unit_norm_store(q, k, eps, k_cache, v_cache, slot_mapping):
+    """q [T,H,D], k [T,G,D] views of a projection output.  Every q head is divided by its root
+    mean square in place; the cache row of a token receives the key before the norm as its VALUE
+    and the key divided by its root mean square as its KEY (D = E).  Rows with slot < 0 store
+    nothing."""
+    qf, kf = q.float(), k.float()
+    q.copy_((qf * torch.rsqrt(qf.pow(2).mean(-1, keepdim=True) + eps)).to(q.dtype))
+    kn = kf * torch.rsqrt(kf.pow(2).mean(-1, keepdim=True) + eps)
+    if k_cache is not None and slot_mapping is not None:
+        bs = k_cache.shape[1]
+        slots = slot_mapping.long()
+        keep = slots >= 0
+        blk, off = torch.div(slots[keep], bs, rounding_mode="floor"), slots[keep] % bs
+        k_cache[blk, off] = kn[keep].to(k_cache.dtype)
+        v_cache[blk, off] = kf[keep].to(v_cache.dtype)
 
 
 # ------------------------------------------------------------------ gated delta rule
@@ -157,7 +188,8 @@ def delta_prepare(q, k, v, b, a, conv_w, a_log, dt_bias, conv_state, cu_q, posit
     """Short causal convolution + silu on q / k / v (their last taps-1 inputs per sequence live
     in ``conv_state`` [slots, taps-1, Cq+Ck+Cv] fp32 and are replaced by this step's), unit
     vectors for q (times D^-1/2) and k, beta = sigmoid(b), decay = exp(-exp(A_log) softplus(a +
-    dt_bias)).  q, k [T,G,D]; v [T,H,E]; b, a [T,H].  Returns fp32 (q, k, v, beta, decay)."""
+    dt_bias)).  q, k [T,G,D]; v [T,H,E]; b [T,H]; a and dt_bias [T,H] / [H] (a decay per head) or
+    [T,H*D] / [H*D] (one per head and key channel).  Returns fp32 (q, k, v, beta, decay)."""
     T, G, D = q.shape
     H, E = v.shape[1], v.shape[2]
     x = torch.cat([q.reshape(T, -1), k.reshape(T, -1), v.reshape(T, -1)], -1).float()
@@ -184,14 +216,19 @@ def delta_prepare(q, k, v, b, a, conv_w, a_log, dt_bias, conv_state, cu_q, posit
     qn = qn * torch.rsqrt(qn.pow(2).sum(-1, keepdim=True) + 1e-6) * D ** -0.5
     kn = kn * torch.rsqrt(kn.pow(2).sum(-1, keepdim=True) + 1e-6)
     beta = torch.sigmoid(b.float())
-    decay = torch.exp(-torch.exp(a_log.float()) * F.softplus(a.float() + dt_bias.float()))
+    sp = F.softplus(a.float() + dt_bias.float())
+    if a.shape[-1] == H:                                                 # one decay per head
+        decay = torch.exp(-torch.exp(a_log.float()) * sp)
+    else:                                                                # one per head and key channel
+        decay = torch.exp(-torch.exp(a_log.float())[None, :, None] * sp.view(T, H, D))
     return qn, kn, vv.contiguous(), beta, decay
 
 
 def delta_scan(qn, kn, vv, beta, decay, state, cu_q, positions, slots):
     """Per sequence and head, token after token: S <- decay S; u = beta (v - S^T k); S <- S + k
     u^T; o = S^T q.  ``state`` [slots, H, D, E] fp32 is read (zeros where the sequence starts at
-    position 0) and left holding the state after the step.  Returns o [T,H,E] fp32."""
+    position 0) and left holding the state after the step.  ``decay`` [T,H] scales a head's whole
+    state, [T,H,D] the rows that belong to key channels.  Returns o [T,H,E] fp32."""
     T, G, D = qn.shape
     H, E = vv.shape[1], vv.shape[2]
     r = H // G
@@ -205,7 +242,7 @@ def delta_scan(qn, kn, vv, beta, decay, state, cu_q, positions, slots):
             continue
         S = state[slot].clone() if int(positions[s]) > 0 else torch.zeros(H, D, E)
         for t in range(s, e):
-            S = S * decay[t][:, None, None]
+            S = S * (decay[t][:, None, None] if decay.dim() == 2 else decay[t][:, :, None])
             u = beta[t][:, None] * (vv[t] - torch.einsum("hde,hd->he", S, kh[t]))
             S = S + kh[t][:, :, None] * u[:, None, :]
             o[t] = torch.einsum("hde,hd->he", S, qh[t])
@@ -213,19 +250,21 @@ def delta_scan(qn, kn, vv, beta, decay, state, cu_q, positions, slots):
     return o
 
 
-def gated_head_norm(o, w, gate, eps, out_dtype):
-    """o [T,H,E] fp32 / rms over E * w[E] * silu(gate [T,H,E])."""
-    y = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * w.float()
-    return (y * F.silu(gate.float()).view(o.shape)).to(out_dtype)
+def gated_head_norm(o, w, gate, eps, out_dtype, act="silu"):
+    """o [T,H,E] fp32 / rms over E * w * act(gate [T,H,E]); w [E] (shared by the heads) or [H*E];
+    act "silu" or "sigmoid"."""
+    y = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * w.float().view(-1, o.shape[-1])
+    gf = gate.float().reshape(o.shape)
+    return (y * (F.silu(gf) if act == "silu" else torch.sigmoid(gf))).to(out_dtype)
 
 
 # ------------------------------------------------------------------ grouped expert routing
-def grouped_route(h, router_w, top, groups, keep):
-    """Softmax over all experts in fp32; only experts of the ``keep`` groups (of ``groups``
+def grouped_route(h, router_w, top, groups, keep, score="softmax"):
+    """Scores over all experts in fp32 (``score``: "softmax", or "sigmoid" of each logit); only experts of the ``keep`` groups (of ``groups``
     equal runs of neighbours) whose best score is largest are eligible; the ``top`` largest
     eligible scores, unnormalised, are the weights.  Returns [T, experts] fp32, zero elsewhere."""
     z = h.float() @ router_w.float().t()
-    s = torch.softmax(z, -1)
+    s = torch.softmax(z, -1) if score == "softmax" else torch.sigmoid(z)
     T, E = s.shape
     per = E // groups
     best = s.view(T, groups, per).max(-1).values
@@ -244,3 +283,121 @@ def gelu_route_scale(up, dense, ff, out_dtype):
     T = up.shape[0]
     y = F.gelu(up.float()).view(T, -1, ff) * dense[:, :, None]
     return y.view(T, -1).to(out_dtype)
+
+
+def swiglu_route_scale(gu, dense, ff, shared_ff, out_dtype):
+    """gu [T, 2 C], C = experts * ff + shared_ff: the gate projections of all experts (and of a
+    shared one behind them), then their up projections.  Column c of expert j gets
+    silu(w g_c) * (w u_c) with w = dense[t, j] - the routing weight scales the expert's INPUT, and
+    the projections are linear, so it is applied to their outputs; exactly zero where w is.
+    Shared columns have w = 1.  ``dense`` None: no routed experts.  Returns [T, C]."""
+    T, C = gu.shape[0], gu.shape[1] // 2
+    g, u = gu[:, :C].float(), gu[:, C:].float()
+    if dense is not None:
+        w = torch.cat([dense.float().repeat_interleave(ff, 1),
+                       torch.ones(T, shared_ff, dtype=torch.float32)], 1)
+        g, u = g * w, u * w
+    return (F.silu(g) * u).to(out_dtype)
+
+
+# ------------------------------------------------------------------ positions, grouped norms
+def embed_sinusoid(ids, positions, table, inv_freq):
+    """fp32 rows ``table[ids]`` + the position vector whose entry 2i is sin(p f_i) and entry
+    2i+1 cos(p f_i); the angle is the fp32 product of the position and ``inv_freq`` [W/2]."""
+    x = table[ids.long()].float()
+    ang = positions.float()[:, None] * inv_freq.float()[None, :]
+    x[:, 0::2] += torch.sin(ang.double()).float()
+    x[:, 1::2] += torch.cos(ang.double()).float()
+    return x
+
+
+def group_rms_norm(x, w, groups, eps, out_dtype):
+    """The row is cut into ``groups`` equal consecutive parts, each divided by its own root mean
+    square; the whole times w."""
+    xf = x.float()
+    parts = xf.view(xf.shape[0], groups, -1)
+    y = parts * torch.rsqrt(parts.pow(2).mean(-1, keepdim=True) + eps)
+    return (y.view(xf.shape) * w.float()).to(out_dtype)
+
+
+def residual_group_norm(x, ys, w_next, groups, eps, out_dtype):
+    """``x += sum(ys)`` in place on the fp32 stream; with ``w_next`` also returns the grouped norm
+    of the new x (the next layer's input)."""
+    for y in ys:
+        x.add_(y.float())
+    if w_next is None:
+        return None
+    return group_rms_norm(x, w_next, groups, eps, out_dtype)
+
+
+def add_normed_mean(x, parts, eps):
+    """``x += mean_i(y_i / rms(y_i) * w_i)`` in place on the fp32 stream; ``parts`` = [(y, w), ...]."""
+    acc = torch.zeros_like(x)
+    for y, w in parts:
+        yf = y.float()
+        acc += yf * torch.rsqrt(yf.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+    x.add_(acc / len(parts))
+
+
+def tanh_cap_(z, cap):
+    """z <- cap tanh(z / cap) in place (fp32 math)."""
+    z.copy_((cap * torch.tanh(z.float() / cap)).to(z.dtype))
+    return z
+
+
+# ------------------------------------------------------------------ gated outer-product recurrences
+def _seq_rows(cu_q, positions, slots):
+    B = slots.shape[0]
+    rows = _bounds(cu_q, positions, B)
+    for i in range(B):
+        s, e, slot = rows[i], rows[i + 1], int(slots[i])
+        if e > s and slot >= 0:
+            yield s, e, slot, int(positions[s]) > 0
+
+
+def mlstm_scan(q, k, v, i_raw, f_raw, i_bias, f_bias, cap, state, norm_state, max_state,
+               cu_q, positions, slots):
+    """Matrix memory with exponential gating and a running maximum m (it starts at 0):
+    i = cap tanh((i_raw + b_i) / cap), f = logsigmoid(cap tanh((f_raw + b_f) / cap)),
+    m' = max(f + m, i); S <- e^(f+m-m') S + e^(i-m') k v^T; n likewise with k alone;
+    o = S^T q / (max(|n . q|, e^(-m')) + 1e-6), q scaled by D^-1/2.  q, k [T,H,D]; v [T,H,E];
+    gates [T,H]; ``state`` [slots,H,D,E], ``norm_state`` [slots,H,D], ``max_state`` [slots,H]
+    fp32.  Returns o [T,H,E] fp32."""
+    T, H, D = q.shape
+    E = v.shape[2]
+    qf, kf, vf = q.float() * D ** -0.5, k.float(), v.float()
+    ig = cap * torch.tanh((i_raw.float() + i_bias.float()) / cap)
+    fg = F.logsigmoid(cap * torch.tanh((f_raw.float() + f_bias.float()) / cap))
+    o = torch.zeros(T, H, E, dtype=torch.float32)
+    for s, e, slot, past in _seq_rows(cu_q, positions, slots):
+        S = state[slot].clone() if past else torch.zeros(H, D, E)
+        n = norm_state[slot].clone() if past else torch.zeros(H, D)
+        m = max_state[slot].clone() if past else torch.zeros(H)
+        for t in range(s, e):
+            m2 = torch.maximum(fg[t] + m, ig[t])
+            a, b = torch.exp(fg[t] + m - m2), torch.exp(ig[t] - m2)
+            S = a[:, None, None] * S + (b[:, None] * kf[t])[:, :, None] * vf[t][:, None, :]
+            n = a[:, None] * n + b[:, None] * kf[t]
+            m = m2
+            den = torch.maximum((n * qf[t]).sum(-1).abs(), torch.exp(-m)) + 1e-6
+            o[t] = torch.einsum("hde,hd->he", S, qf[t]) / den[:, None]
+        state[slot], norm_state[slot], max_state[slot] = S, n, m
+    return o
+
+
+def gla_scan(q, k, v, a_raw, a_bias, tau, state, cu_q, positions, slots):
+    """S <- diag(alpha) S + k v^T; o = S^T q with alpha = sigmoid(a_raw + a_bias)^(1/tau) per key
+    channel (rows of S) and q scaled by D^-1/2.  q, k, a_raw [T,H,D]; v [T,H,E]; ``state``
+    [slots,H,D,E] fp32.  Returns o [T,H,E] fp32."""
+    T, H, D = q.shape
+    E = v.shape[2]
+    qf, kf, vf = q.float() * D ** -0.5, k.float(), v.float()
+    alpha = torch.exp(F.logsigmoid(a_raw.float().reshape(T, H, D) + a_bias.float().view(H, D)) / tau)
+    o = torch.zeros(T, H, E, dtype=torch.float32)
+    for s, e, slot, past in _seq_rows(cu_q, positions, slots):
+        S = state[slot].clone() if past else torch.zeros(H, D, E)
+        for t in range(s, e):
+            S = alpha[t][:, :, None] * S + kf[t][:, :, None] * vf[t][:, None, :]
+            o[t] = torch.einsum("hde,hd->he", S, qf[t])
+        state[slot] = S
+    return o
