@@ -13,9 +13,35 @@
 // starts at the sink and the running sum at 1 = exp(sink - sink): the sink is a key without a
 // value.  Rows: a decode batch (row b = sequence b, context_lens[b] keys) or the rows of a
 // prefill-form step (row_seq gives the sequence, positions[t] + 1 keys).
+//
+// Options of all three (struct KeyRule): no sink (sink == null: an ordinary softmax; the running
+// maximum then starts at a large negative FINITE number and the sum at 0, so that no path forms
+// inf - inf), a sliding window that keeps the first tokens (a query at position i sees key j <= i
+// only when i - j < window or j < keep_first; keys outside are never loaded), and a distance
+// penalty slope_h * (i - j) taken off the score.
 #include "hybrid_common.h"
 
 using namespace hyb;
+
+constexpr float NO_SINK_MAX = -1e30f;
+
+struct KeyRule {
+    int window;             // 0: every earlier key is visible
+    int keep_first;
+    const float* slopes;    // [H] or null
+};
+
+// The visible keys of a query that sees `ctx` keys without a window (its position is ctx - 1), as
+// one run of virtual indices: [0, kept) are keys 0 .. kept-1, the rest the window's keys from `lo`.
+struct VisibleKeys {
+    int kept, lo, count;
+    __device__ __forceinline__ VisibleKeys(int ctx, const KeyRule& r) {
+        lo = r.window > 0 ? max(0, ctx - r.window) : 0;
+        kept = min(r.keep_first, lo);
+        count = kept + ctx - lo;
+    }
+    __device__ __forceinline__ int key(int v) const { return v < kept ? v : lo + (v - kept); }
+};
 
 constexpr int TILE = 256;
 constexpr int RC = 4;       // query heads per workgroup
@@ -29,7 +55,8 @@ sink_attention_rows_kernel(const T* __restrict__ q, long q_row, long q_head,
                            const int* __restrict__ row_seq, const int* __restrict__ lens,
                            int len_add, const float* __restrict__ sink,
                            const T* __restrict__ gate, long gate_row, T* __restrict__ out,
-                           float scale, int H, int G, int D, int E, int vec_ok, int seq_base) {
+                           float scale, int H, int G, int D, int E, int vec_ok, int seq_base,
+                           KeyRule rule) {
     extern __shared__ float sm[];
     const int R = H / G;
     const int chunks = (R + RC - 1) / RC;
@@ -40,6 +67,7 @@ sink_attention_rows_kernel(const T* __restrict__ q, long q_row, long q_head,
     if (b < 0) return;
     const int ctx = lens[row_seq ? t : b] + len_add;
     if (ctx <= 0) return;
+    const VisibleKeys vis(ctx, rule);
     const int* table = block_tables + (long)b * max_blocks;
     const int tid = threadIdx.x, wave = tid / kWave, lane = tid & (kWave - 1);
 
@@ -54,17 +82,20 @@ sink_attention_rows_kernel(const T* __restrict__ q, long q_row, long q_head,
         qs[r * D + d] = ld(q + t * q_row + (long)(h0 + r) * q_head + d) * scale;
     }
     if (tid < RC) {
-        stat[RC + tid] = tid < nr ? sink[h0 + tid] : 0.f;       // running max
-        stat[2 * RC + tid] = 1.f;                               // running sum (the sink's term)
+        stat[RC + tid] = tid < nr ? (sink ? sink[h0 + tid] : NO_SINK_MAX) : 0.f;   // running max
+        stat[2 * RC + tid] = sink ? 1.f : 0.f;                  // running sum (the sink's term)
     }
+    float slope[RC];
+#pragma unroll
+    for (int r = 0; r < RC; ++r) slope[r] = (rule.slopes && r < nr) ? rule.slopes[h0 + r] : 0.f;
     float acc[NACC];
 #pragma unroll
     for (int a = 0; a < NACC; ++a) acc[a] = 0.f;
     __syncthreads();
 
-    for (int j0 = 0; j0 < ctx; j0 += TILE) {
-        const int j = j0 + tid;
-        const bool live = j < ctx;
+    for (int j0 = 0; j0 < vis.count; j0 += TILE) {
+        const bool live = j0 + tid < vis.count;
+        const int j = vis.key(j0 + tid);
         float s[RC];
 #pragma unroll
         for (int r = 0; r < RC; ++r) s[r] = -INFINITY;
@@ -92,6 +123,9 @@ sink_attention_rows_kernel(const T* __restrict__ q, long q_row, long q_head,
                     for (int r = 0; r < RC; ++r) if (r < nr) s[r] += kv * qs[r * D + d];
                 }
             }
+            const float dist = (float)(ctx - 1 - j);
+#pragma unroll
+            for (int r = 0; r < RC; ++r) s[r] -= slope[r] * dist;
         }
         // tile maximum per head
 #pragma unroll
@@ -129,7 +163,7 @@ sink_attention_rows_kernel(const T* __restrict__ q, long q_row, long q_head,
         }
         __syncthreads();
         // weighted value sums: thread owns columns c = tid + a * TILE of [nr][E]
-        const int n = min(TILE, ctx - j0);
+        const int n = min(TILE, vis.count - j0);
 #pragma unroll
         for (int a = 0; a < NACC; ++a) {
             const int c = tid + a * TILE;
@@ -184,7 +218,7 @@ sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
                             const int* __restrict__ cu_q, const int* __restrict__ positions,
                             const float* __restrict__ sink, const T* __restrict__ gate,
                             long gate_row, T* __restrict__ out, float scale, int H, int G, int D,
-                            int E, int seq0, int vec_k, int vec_v) {
+                            int E, int seq0, int vec_k, int vec_v, KeyRule rule) {
     extern __shared__ float sm[];
     constexpr int KS = QK16 ? (DP + 8) / 2 : DP + 1;      // floats per K row of the LDS image
     constexpr int KSB = DP + 8;                             // (QK16) 16-bit elements per K row
@@ -230,7 +264,8 @@ sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
             }
         }
     }
-    float m = sink[h], lsum = 1.f;
+    float m = sink ? sink[h] : NO_SINK_MAX, lsum = sink ? 1.f : 0.f;
+    const float slope = rule.slopes ? rule.slopes[h] : 0.f;
     f32x16 oacc[EP / 32];
 #pragma unroll
     for (int eb = 0; eb < EP / 32; ++eb)
@@ -240,8 +275,12 @@ sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
     const int wg_ctx = start + min(qlen, tile * 128 + 128);            // keys this workgroup needs
     const bool wave_live = tile * 128 + wave * 32 < qlen;
     const int wave_last = start + min(qlen - 1, tile * 128 + wave * 32 + 31);
+    // with a window: the oldest key any query of the workgroup / of the wave still sees
+    const int wg_lo = rule.window > 0 ? max(0, start + tile * 128 - rule.window + 1) : 0;
+    const int wave_lo = rule.window > 0 ? max(0, start + tile * 128 + wave * 32 - rule.window + 1) : 0;
 
     for (int k0 = 0; k0 < wg_ctx; k0 += 32) {
+        if (k0 >= rule.keep_first && k0 + 32 <= wg_lo) continue;     // (uniform) nobody sees this tile
         // ---- K and V tile into LDS
         if constexpr (QK16) {
             const int D8 = D >> 3;
@@ -301,7 +340,7 @@ sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
             }
         }
         __syncthreads();
-        if (wave_live && k0 <= wave_last) {
+        if (wave_live && k0 <= wave_last && (k0 < rule.keep_first || k0 + 32 > wave_lo)) {
             f32x16 sacc;
 #pragma unroll
             for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
@@ -324,7 +363,9 @@ sink_attention_tiles_kernel(const T* __restrict__ q, long q_row, long q_head,
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int key = k0 + 8 * (r >> 2) + 4 * half + (r & 3);
-                const float v = (qok && key <= qpos) ? sacc[r] : -INFINITY;
+                const bool seen = qok && key <= qpos &&
+                                  (rule.window <= 0 || qpos - key < rule.window || key < rule.keep_first);
+                const float v = seen ? sacc[r] - slope * (float)(qpos - key) : -INFINITY;
                 sacc[r] = v;
                 mt = fmaxf(mt, v);
             }
@@ -374,7 +415,7 @@ static int launch_tiles(const void* q, long q_row, long q_head, const void* k_ca
                         int block_size, const void* cu_q, const void* positions, const void* sink,
                         const void* gate, long gate_row, void* out, float scale, int nseq,
                         int seq0, int max_q, int H, int G, int D, int E, int esize,
-                        hipStream_t s) {
+                        KeyRule rule, hipStream_t s) {
     const int vec_k = (D % 4 == 0) && ((size_t)k_cache % 16 == 0);
     const int vec_v = (E % 4 == 0) && ((size_t)v_cache % 16 == 0);
     const dim3 grid(nseq, (max_q + 127) / 128, H);
@@ -383,7 +424,7 @@ static int launch_tiles(const void* q, long q_row, long q_head, const void* k_ca
                        (const T*)q, q_row, q_head, (const T*)k_cache, (const T*)v_cache,          \
                        (const int*)block_tables, max_blocks, block_size, (const int*)cu_q,        \
                        (const int*)positions, (const float*)sink, (const T*)gate, gate_row,       \
-                       (T*)out, scale, H, G, D, E, seq0, vec_k, vec_v)
+                       (T*)out, scale, H, G, D, E, seq0, vec_k, vec_v, rule)
     if constexpr (sizeof(T) == 2) {
         // 16-bit caches: score products on the bf16 instruction when rows are 16-byte addressable
         if (D % 16 == 0 && (size_t)k_cache % 16 == 0 && (size_t)q % 16 == 0 && q_row % 8 == 0 &&
@@ -411,7 +452,8 @@ sink_attention_split_kernel(const T* __restrict__ q, long q_row, long q_head,
                             const T* __restrict__ k_cache, const T* __restrict__ v_cache,
                             const int* __restrict__ block_tables, int max_blocks, int block_size,
                             const int* __restrict__ context_lens, const float* __restrict__ sink,
-                            float* __restrict__ ws, float scale, int H, int G, int splits) {
+                            float* __restrict__ ws, float scale, int H, int G, int splits,
+                            KeyRule rule) {
     constexpr int D = 16 * EPL, E = 16 * VPL;
     extern __shared__ float sm[];                 // [16 groups][RC][E + 2]
     const int R = H / G, chunks = (R + RC - 1) / RC;
@@ -420,31 +462,35 @@ sink_attention_split_kernel(const T* __restrict__ q, long q_row, long q_head,
     const int nr = min(RC, g * R + R - h0);
     const int ctx = context_lens[b];
     const int tid = threadIdx.x, lane16 = tid & 15, kg = tid >> 4;
-    const int span = ((ctx + splits - 1) / splits + 15) & ~15;
-    const int k_begin = split * span, k_end = min(ctx, k_begin + span);
+    const VisibleKeys vis(ctx, rule);
+    const int span = ((vis.count + splits - 1) / splits + 15) & ~15;
+    const int k_begin = split * span, k_end = min(vis.count, k_begin + span);
     const int* table = block_tables + (long)b * max_blocks;
 
-    float qf[RC][EPL], m[RC], l[RC], acc[RC][VPL];
+    float qf[RC][EPL], m[RC], l[RC], acc[RC][VPL], slope[RC];
 #pragma unroll
     for (int r = 0; r < RC; ++r) {
         if (r < nr) {
             load_run<T, EPL>(q + b * q_row + (long)(h0 + r) * q_head + lane16 * EPL, qf[r]);
 #pragma unroll
             for (int i = 0; i < EPL; ++i) qf[r][i] *= scale;
-            m[r] = sink[h0 + r];
+            m[r] = sink ? sink[h0 + r] : NO_SINK_MAX;
+            slope[r] = rule.slopes ? rule.slopes[h0 + r] : 0.f;
         } else {
 #pragma unroll
             for (int i = 0; i < EPL; ++i) qf[r][i] = 0.f;
             m[r] = 0.f;
+            slope[r] = 0.f;
         }
         l[r] = 0.f;
 #pragma unroll
         for (int i = 0; i < VPL; ++i) acc[r][i] = 0.f;
     }
     // two keys per trip: both rows' loads are in flight before the first one is used
-    for (int j = k_begin + kg; j < k_end; j += 32) {
-        const int j2 = j + 16;
-        const bool two = j2 < k_end;
+    for (int vj = k_begin + kg; vj < k_end; vj += 32) {
+        const bool two = vj + 16 < k_end;
+        const int j = vis.key(vj), j2 = two ? vis.key(vj + 16) : j;
+        const float dist[2] = {(float)(ctx - 1 - j), (float)(ctx - 1 - j2)};
         const long slot = (long)table[j / block_size] * block_size + j % block_size;
         const long slot2 = two ? (long)table[j2 / block_size] * block_size + j2 % block_size : slot;
         float kf[2][EPL], vf[2][VPL];
@@ -465,6 +511,7 @@ sink_attention_split_kernel(const T* __restrict__ q, long q_row, long q_head,
                 d += __shfl_xor(d, 2, kWave);
                 d += __shfl_xor(d, 4, kWave);
                 d += __shfl_xor(d, 8, kWave);
+                d -= slope[r] * dist[x];
                 if (d > m[r]) {                    // the running maximum moves: rescale (rare)
                     const float a = expf(m[r] - d);
                     l[r] *= a;
@@ -516,9 +563,9 @@ __global__ void sink_attention_merge_kernel(const float* __restrict__ ws,
     if (context_lens[b] <= 0) return;
     const int PS = E + 2;
     const float* p = ws + ((long)b * H + h) * splits * PS;
-    float M = sink[h];
+    float M = sink ? sink[h] : NO_SINK_MAX;
     for (int s = 0; s < splits; ++s) M = fmaxf(M, p[s * PS]);
-    float L = expf(sink[h] - M);
+    float L = sink ? expf(sink[h] - M) : 0.f;
     for (int s = 0; s < splits; ++s) L += p[s * PS + 1] * expf(p[s * PS] - M);
     float f = 1.f / L;
     if (gate) f *= sigmoidf_(ld(gate + b * gate_row + h));
@@ -534,14 +581,15 @@ static int launch_split(const void* q, long q_row, long q_head, const void* k_ca
                         const void* v_cache, const void* block_tables, int max_blocks,
                         int block_size, const void* context_lens, const void* sink,
                         const void* gate, long gate_row, void* out, void* ws, float scale, int B,
-                        int H, int G, int splits, hipStream_t s) {
+                        int H, int G, int splits, KeyRule rule, hipStream_t s) {
     constexpr int E = 16 * VPL;
     const int R = H / G, chunks = (R + RC - 1) / RC;
     const size_t lds = 16 * RC * (E + 2) * sizeof(float);
     hipLaunchKernelGGL((sink_attention_split_kernel<T, EPL, VPL>), dim3(B, G * chunks, splits),
                        dim3(256), lds, s, (const T*)q, q_row, q_head, (const T*)k_cache,
                        (const T*)v_cache, (const int*)block_tables, max_blocks, block_size,
-                       (const int*)context_lens, (const float*)sink, (float*)ws, scale, H, G, splits);
+                       (const int*)context_lens, (const float*)sink, (float*)ws, scale, H, G, splits,
+                       rule);
     if (hipGetLastError() != hipSuccess) return 2;
     hipLaunchKernelGGL(sink_attention_merge_kernel<T>, dim3(B * H), dim3(E >= 128 ? 128 : 64), 0, s,
                        (const float*)ws, (const float*)sink, (const T*)gate, gate_row,
@@ -561,12 +609,14 @@ int hyb_sink_attention_split(const void* q, long q_row, long q_head, const void*
                              const void* v_cache, const void* block_tables, int max_blocks,
                              int block_size, const void* context_lens, const void* sink,
                              const void* gate, long gate_row, void* out, void* ws, float scale,
-                             int B, int H, int G, int D, int E, int splits, int dt, hipStream_t s) {
+                             int B, int H, int G, int D, int E, int splits, int window,
+                             int keep_first, const void* slopes, int dt, hipStream_t s) {
+    const KeyRule rule{window, keep_first, (const float*)slopes};
     if (B <= 0) return 0;
     if (G <= 0 || H % G || splits < 1 || !hyb_sink_attention_split_ok(D, E)) return 1;
     if (((size_t)k_cache | (size_t)v_cache | (size_t)q) % 16 || (q_row * (dt == 0 ? 2 : 4)) % 16) return 1;
 #define SPLIT_ARGS q, q_row, q_head, k_cache, v_cache, block_tables, max_blocks, block_size, \
-                   context_lens, sink, gate, gate_row, out, ws, scale, B, H, G, splits, s
+                   context_lens, sink, gate, gate_row, out, ws, scale, B, H, G, splits, rule, s
 #define SPLIT_E(T, EPL)                                                  \
     do {                                                                 \
         if (E == 64) return launch_split<T, EPL, 4>(SPLIT_ARGS);         \
@@ -593,16 +643,18 @@ int hyb_sink_attention_tiles(const void* q, long q_row, long q_head, const void*
                              int block_size, const void* cu_q, const void* positions,
                              const void* sink, const void* gate, long gate_row, void* out,
                              float scale, int nseq, int seq0, int max_q, int H, int G, int D,
-                             int E, int dt, hipStream_t s) {
+                             int E, int window, int keep_first, const void* slopes, int dt,
+                             hipStream_t s) {
+    const KeyRule rule{window, keep_first, (const float*)slopes};
     if (nseq <= 0 || max_q <= 0) return 0;
     if (G <= 0 || H % G || !hyb_sink_attention_tiles_ok(D, E)) return 1;
 #define TILES_ARGS q, q_row, q_head, k_cache, v_cache, block_tables, max_blocks, block_size, cu_q, \
                    positions, sink, gate, gate_row, out, scale, nseq, seq0, max_q, H, G, D, E
 #define TILES_E(T, DP, esz)                                                   \
     do {                                                                      \
-        if (E <= 64) return launch_tiles<T, DP, 64>(TILES_ARGS, esz, s);      \
-        if (E <= 128) return launch_tiles<T, DP, 128>(TILES_ARGS, esz, s);    \
-        if (DP <= 128) return launch_tiles<T, (DP <= 128 ? DP : 64), 256>(TILES_ARGS, esz, s); \
+        if (E <= 64) return launch_tiles<T, DP, 64>(TILES_ARGS, esz, rule, s);      \
+        if (E <= 128) return launch_tiles<T, DP, 128>(TILES_ARGS, esz, rule, s);    \
+        if (DP <= 128) return launch_tiles<T, (DP <= 128 ? DP : 64), 256>(TILES_ARGS, esz, rule, s); \
         return 1;                                                             \
     } while (0)
 #define TILES_D(T, esz)                                   \
@@ -623,7 +675,8 @@ int hyb_sink_attention_rows(const void* q, long q_row, long q_head, const void* 
                             int block_size, const void* row_seq, const void* lens, int len_add,
                             const void* sink, const void* gate, long gate_row, void* out,
                             float scale, long rows, int H, int G, int D, int E, int seq_base,
-                            int dt, hipStream_t s) {
+                            int window, int keep_first, const void* slopes, int dt, hipStream_t s) {
+    const KeyRule rule{window, keep_first, (const float*)slopes};
     if (rows <= 0) return 0;
     if (G <= 0 || H % G || RC * E > NACC * TILE || D > 1024) return 1;
     const int R = H / G, chunks = (R + RC - 1) / RC;
@@ -636,7 +689,7 @@ int hyb_sink_attention_rows(const void* q, long q_row, long q_head, const void* 
                                         (const int*)block_tables, max_blocks, block_size,
                                         (const int*)row_seq, (const int*)lens, len_add,
                                         (const float*)sink, (const T*)gate, gate_row, (T*)out,
-                                        scale, H, G, D, E, vec_ok, seq_base));
+                                        scale, H, G, D, E, vec_ok, seq_base, rule));
     return HYB_LAUNCH_OK();
 }
 

@@ -12,12 +12,16 @@ using namespace hyb;
 
 constexpr int MAX_TAPS = 32;
 
-// One workgroup per token row.  proj row = [q (G*D) | k (G*D) | v (H*E) | gate | b (H) | a (H)];
-// the three convolved blocks are contiguous at the row's start (C = 2GD + HE channels).
+// One workgroup per token row.  proj row = [q (G*D) | k (G*D) | v (H*E) | ... | b (H) | ...];
+// the three convolved blocks are contiguous at the row's start (C = 2GD + HE channels).  The
+// decay's pre-activation `a` is a row of its own tensor (or a view into proj): DC entries per
+// head, DC = 1 (a decay per head) or D (one per head and key channel); dt_bias has H * DC
+// entries, decay out [T, H * DC].
 // conv_w [C, taps] (q, k, v rows stacked), conv_state [slots, taps-1, C].
 template <typename T, int TAPS>
 __global__ void delta_prepare_kernel(const T* __restrict__ proj, long row_stride, int b_off,
-                                     int a_off, const float* __restrict__ conv_w, int taps_rt,
+                                     const T* __restrict__ a, long a_row, int DC,
+                                     const float* __restrict__ conv_w, int taps_rt,
                                      const float* __restrict__ a_log,
                                      const float* __restrict__ dt_bias,
                                      const float* __restrict__ conv_state,
@@ -97,10 +101,11 @@ __global__ void delta_prepare_kernel(const T* __restrict__ proj, long row_stride
         else dst = kn + (t * G + hd - G) * (long)D;
         for (int d = lane; d < D; d += kWave) dst[d] = src[d] * r;
     }
-    for (int h = threadIdx.x; h < H; h += blockDim.x) {
+    for (int h = threadIdx.x; h < H; h += blockDim.x)
         beta[t * H + h] = sigmoidf_(ld(proj + t * row_stride + b_off + h));
-        const float z = ld(proj + t * row_stride + a_off + h) + dt_bias[h];
-        decay[t * H + h] = expf(-expf(a_log[h]) * softplusf_(z));
+    for (int c = threadIdx.x; c < H * DC; c += blockDim.x) {
+        const float z = ld(a + t * a_row + c) + dt_bias[c];
+        decay[t * (long)(H * DC) + c] = expf(-expf(a_log[c / DC]) * softplusf_(z));
     }
 }
 
@@ -281,13 +286,13 @@ static void launch_scan(dim3 grid, hipStream_t s, const void* qn, const void* kn
 
 extern "C" {
 
-int hyb_delta_prepare(const void* proj, long row_stride, int b_off, int a_off, const void* conv_w,
-                      int taps, const void* a_log, const void* dt_bias, void* conv_state,
+int hyb_delta_prepare(const void* proj, long row_stride, int b_off, const void* a, long a_row,
+                      int DC, const void* conv_w, int taps, const void* a_log, const void* dt_bias, void* conv_state,
                       const void* cu_q, const void* positions, const void* slots,
                       const void* row_seq, void* qn, void* kn, void* vv, void* beta, void* decay,
                       long T_, int B, int H, int G, int D, int E, int dt, hipStream_t s) {
     if (T_ <= 0) return 0;
-    if (taps < 1 || taps > MAX_TAPS || H % G) return 1;
+    if (taps < 1 || taps > MAX_TAPS || H % G || (DC != 1 && DC != D)) return 1;
     const int C = 2 * G * D + H * E;
     const size_t lds = 2 * (size_t)G * D * sizeof(float);
     if (lds > 64 * 1024) return 1;
@@ -296,7 +301,7 @@ int hyb_delta_prepare(const void* proj, long row_stride, int b_off, int a_off, c
 #define PREP(TAPS)                                                                                 \
     HYB_DISPATCH(dt, hipLaunchKernelGGL((delta_prepare_kernel<T, TAPS>), dim3(T_),                 \
                                         dim3(C >= 2048 && T_ <= 1024 ? 1024 : 256), lds, s,        \
-                                        (const T*)proj, row_stride, b_off, a_off,                  \
+                                        (const T*)proj, row_stride, b_off, (const T*)a, a_row, DC, \
                                         (const float*)conv_w, taps, (const float*)a_log,           \
                                         (const float*)dt_bias, (const float*)conv_state,           \
                                         (const int*)cu_q, (const int*)positions, (const int*)slots,\

@@ -108,11 +108,13 @@ __global__ void pair_rope_mix_store_kernel(T* __restrict__ q, const T* __restric
     }
 }
 
-// out[t,h,:] = o[t,h,:] / rms(o[t,h,:]) * w * silu(gate[t,h,:]); one wave per (t, h)
+// out[t,h,:] = o[t,h,:] / rms(o[t,h,:]) * w * act(gate[t,h,:]); one wave per (t, h).  w_heads: w
+// has H * E entries (0: E entries shared by the heads); sig: act is the sigmoid (0: silu).
 template <typename T>
 __global__ void gated_head_norm_kernel(const float* __restrict__ o, const float* __restrict__ w,
                                        const T* __restrict__ gate, long gate_stride,
-                                       T* __restrict__ out, int H, int E, float eps) {
+                                       T* __restrict__ out, int H, int E, float eps, int w_heads,
+                                       int sig) {
     const long th = blockIdx.x;
     const long t = th / H;
     const int h = th - t * H;
@@ -121,18 +123,21 @@ __global__ void gated_head_norm_kernel(const float* __restrict__ o, const float*
     for (int e = threadIdx.x; e < E; e += kWave) { const float v = orow[e]; s += v * v; }
     const float r = rsqrtf(wave_sum(s) / (float)E + eps);
     const T* g = gate + t * gate_stride + (long)h * E;
-    for (int e = threadIdx.x; e < E; e += kWave)
-        st(out + th * E + e, orow[e] * r * w[e] * siluf_(ld(g + e)));
+    const float* wh = w + (w_heads ? (long)h * E : 0);
+    for (int e = threadIdx.x; e < E; e += kWave) {
+        const float z = ld(g + e);
+        st(out + th * E + e, orow[e] * r * wh[e] * (sig ? sigmoidf_(z) : siluf_(z)));
+    }
 }
 
 // One workgroup (256 threads) per token: fp32 router logits (the row is read once, eight experts'
-// partial sums per pass), softmax over all experts, best `keep` of `groups` groups (a group
+// partial sums per pass), softmax over all experts (sig: sigmoid of each logit), best `keep` of `groups` groups (a group
 // scores its best expert), `top` largest eligible scores; dense [T, NE] out, zero where not
 // chosen.  Ties go to the lower index.  LDS: 2 * NE + 32 floats.
 template <typename T>
 __global__ void grouped_route_kernel(const T* __restrict__ h, const float* __restrict__ wr,
                                      float* __restrict__ dense, int W, int NE, int top,
-                                     int groups, int keep) {
+                                     int groups, int keep, int sig) {
     extern __shared__ float sm[];
     float* z = sm;              // scores
     float* elig = sm + NE;      // eligible scores (or -1)
@@ -165,7 +170,13 @@ __global__ void grouped_route_kernel(const T* __restrict__ h, const float* __res
         }
         __syncthreads();
     }
-    if (threadIdx.x < kWave) {
+    if (threadIdx.x < kWave && sig) {            // every expert scored by the sigmoid of its own logit
+        for (int e = threadIdx.x; e < NE; e += kWave) {
+            z[e] = sigmoidf_(z[e]);
+            elig[e] = -1.f;
+            dense[t * NE + e] = 0.f;
+        }
+    } else if (threadIdx.x < kWave) {
         float m = -INFINITY;
         for (int e = threadIdx.x; e < NE; e += kWave) m = fmaxf(m, z[e]);
         m = wave_max(m);
@@ -271,21 +282,22 @@ int hyb_pair_rope_mix_store(void* q, const void* k, const void* v, long row_stri
 }
 
 int hyb_gated_head_norm(const void* o, const void* w, const void* gate, long gate_stride,
-                        void* out, long T_, int H, int E, float eps, int dt, hipStream_t s) {
+                        void* out, long T_, int H, int E, float eps, int w_heads, int sig, int dt,
+                        hipStream_t s) {
     if (T_ <= 0) return 0;
     HYB_DISPATCH(dt, hipLaunchKernelGGL(gated_head_norm_kernel<T>, dim3(T_ * H), dim3(kWave), 0, s,
                                         (const float*)o, (const float*)w, (const T*)gate,
-                                        gate_stride, (T*)out, H, E, eps));
+                                        gate_stride, (T*)out, H, E, eps, w_heads, sig));
     return HYB_LAUNCH_OK();
 }
 
 int hyb_grouped_route(const void* h, const void* wr, void* dense, long T_, int W, int NE, int top,
-                      int groups, int keep, int dt, hipStream_t s) {
+                      int groups, int keep, int sig, int dt, hipStream_t s) {
     if (T_ <= 0) return 0;
     if (groups <= 0 || NE % groups || keep > groups || top > NE / groups * keep || NE > 4096) return 1;
     HYB_DISPATCH(dt, hipLaunchKernelGGL(grouped_route_kernel<T>, dim3(T_), dim3(256),
                                         (2 * NE + 32) * sizeof(float), s, (const T*)h, (const float*)wr,
-                                        (float*)dense, W, NE, top, groups, keep));
+                                        (float*)dense, W, NE, top, groups, keep, sig));
     return HYB_LAUNCH_OK();
 }
 

@@ -35,24 +35,35 @@ _norm = _sig("hyb_offset_rms_norm", _P, _P, _P, _L, _I, _F, _I, _P)
 _post = _sig("hyb_post_norm_residual", _P, _L, _P, _P, _P, _P, _L, _I, _F, _I, _P)
 _rope = _sig("hyb_pair_rope_mix_store", _P, _P, _P, _L, _P, _P, _I, _P, _P, _I, _P, _P, _P, _L,
              _I, _I, _I, _I, _I, _P)
-_ghn = _sig("hyb_gated_head_norm", _P, _P, _P, _L, _P, _L, _I, _I, _F, _I, _P)
-_route = _sig("hyb_grouped_route", _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _P)
+_ghn = _sig("hyb_gated_head_norm", _P, _P, _P, _L, _P, _L, _I, _I, _F, _I, _I, _I, _P)
+_route = _sig("hyb_grouped_route", _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _I, _P)
 _gelu = _sig("hyb_gelu_route_scale", _P, _P, _P, _L, _I, _I, _I, _P)
 _attn = _sig("hyb_sink_attention_rows", _P, _L, _L, _P, _P, _P, _I, _I, _P, _P, _I, _P, _P, _L, _P,
-             _F, _L, _I, _I, _I, _I, _I, _I, _P)
+             _F, _L, _I, _I, _I, _I, _I, _I, _I, _P, _I, _P)
 _tiles = _sig("hyb_sink_attention_tiles", _P, _L, _L, _P, _P, _P, _I, _I, _P, _P, _P, _P, _L, _P, _F,
-              _I, _I, _I, _I, _I, _I, _I, _I, _P)
+              _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _I, _P)
 _tiles_ok = _lib.hyb_sink_attention_tiles_ok
 _tiles_ok.argtypes = [_I, _I]
 _tiles_ok.restype = _I
 _split = _sig("hyb_sink_attention_split", _P, _L, _L, _P, _P, _P, _I, _I, _P, _P, _P, _L, _P, _P, _F,
-              _I, _I, _I, _I, _I, _I, _I, _P)
+              _I, _I, _I, _I, _I, _I, _I, _I, _P, _I, _P)
 _split_ok = _lib.hyb_sink_attention_split_ok
 _split_ok.argtypes = [_I, _I]
 _split_ok.restype = _I
-_prep = _sig("hyb_delta_prepare", _P, _L, _I, _I, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P,
-             _P, _P, _L, _I, _I, _I, _I, _I, _I, _P)
+_prep = _sig("hyb_delta_prepare", _P, _L, _I, _P, _L, _I, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P,
+             _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _P)
 _scan = _sig("hyb_delta_scan", _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P)
+_cscan = _sig("hyb_channel_delta_scan", _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P)
+_gla = _sig("hyb_gla_scan", _P, _P, _P, _L, _L, _L, _P, _L, _P, _F, _P, _P, _P, _P, _P, _I, _I, _I, _I,
+            _I, _P)
+_mlstm = _sig("hyb_mlstm_scan", _P, _P, _P, _L, _L, _L, _P, _P, _L, _P, _P, _F, _P, _P, _P, _P, _P, _P,
+              _P, _I, _I, _I, _I, _I, _P)
+_esin = _sig("hyb_embed_sinusoid", _P, _P, _P, _P, _P, _L, _I, _I, _P)
+_rgn = _sig("hyb_residual_group_norm", _P, _P, _L, _P, _L, _P, _P, _L, _I, _I, _F, _I, _P)
+_anm = _sig("hyb_add_normed_mean", _P, _P, _L, _P, _P, _L, _P, _L, _I, _F, _I, _P)
+_uns = _sig("hyb_unit_norm_store", _P, _P, _L, _F, _P, _P, _P, _L, _I, _I, _I, _I, _P)
+_swi = _sig("hyb_swiglu_route_scale", _P, _L, _P, _P, _L, _I, _I, _I, _I, _P)
+_cap = _sig("hyb_tanh_cap", _P, _L, _F, _I, _P)
 
 _DT = {torch.bfloat16: 0, torch.float32: 2}
 
@@ -148,8 +159,15 @@ def pair_rope_mix_store(q, k, v, positions, cos_sin, rot_dims, v_first, lam, v_m
 
 
 # ------------------------------------------------------------------ attention with a sink
+def _slopes(slopes, H):
+    if slopes is None:
+        return None
+    assert slopes.dtype == torch.float32 and slopes.is_contiguous() and slopes.numel() == H
+    return slopes.data_ptr()
+
+
 def _attention_rows(q, k_cache, v_cache, block_tables, row_seq, lens, len_add, scale, sink, gate, out,
-                    seq_base=0):
+                    seq_base=0, window=0, keep_first=0, slopes=None):
     T, H, D = q.shape
     G, E = k_cache.shape[2], v_cache.shape[3]
     assert q.stride(2) == 1 and out.is_contiguous() and out.shape == (T, H, E) and out.dtype == q.dtype
@@ -159,23 +177,26 @@ def _attention_rows(q, k_cache, v_cache, block_tables, row_seq, lens, len_add, s
         assert gate.stride(1) == 1 and gate.dtype == q.dtype
     _check(_attn(q.data_ptr(), q.stride(0), q.stride(1), k_cache.data_ptr(), v_cache.data_ptr(),
                  block_tables.data_ptr(), block_tables.stride(0), k_cache.shape[1],
-                 _ptr(_i32(row_seq)), _i32(lens).data_ptr(), len_add, _f32(sink).data_ptr(),
+                 _ptr(_i32(row_seq)), _i32(lens).data_ptr(), len_add,
+                 _f32(sink).data_ptr() if sink is not None else None,
                  _ptr(gate), gate.stride(0) if gate is not None else 0, out.data_ptr(), scale, T,
-                 H, G, D, E, seq_base, _dt(q), _stream()), "sink_attention")
+                 H, G, D, E, seq_base, int(window), int(keep_first), _slopes(slopes, H), _dt(q),
+                 _stream()), "sink_attention")
     return out
 
 
 def sink_attention_step(q, k_cache, v_cache, block_tables, row_seq, positions, scale, sink, gate, out,
-                        seq_base=0):
+                        seq_base=0, window=0, keep_first=0, slopes=None):
     """Rows of a prefill-form step, one workgroup per row: row t belongs to sequence
     ``row_seq[t]`` (< ``seq_base``: skipped), whose block table is row ``row_seq[t] - seq_base``
     of ``block_tables``, and sees ``positions[t] + 1`` keys."""
     return _attention_rows(q, k_cache, v_cache, block_tables, row_seq, positions, 1, scale, sink,
-                           gate, out, seq_base)
+                           gate, out, seq_base, window, keep_first, slopes)
 
 
 def sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables, scale, sink, gate, out,
-                           positions=None, max_q=None, row_seq=None, first_seq=0):
+                           positions=None, max_q=None, row_seq=None, first_seq=0,
+                           window=0, keep_first=0, slopes=None):
     """The prompt portions of a step: sequence b owns rows cu_q[b] .. cu_q[b+1] (absolute rows
     of q / out / positions) and block table row b.  Runs the matrix-core tile kernel (fp32
     scores, weights and sums); head sizes it has no instance for go row by row.  ``cu_k`` is
@@ -188,7 +209,8 @@ def sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables, scale,
         assert row_seq is not None
         # ``first_seq``: number of the step's sequences ahead of these (its decode riders)
         return sink_attention_step(q, k_cache, v_cache, block_tables, row_seq, positions, scale,
-                                   sink, gate, out, seq_base=first_seq)
+                                   sink, gate, out, seq_base=first_seq, window=window,
+                                   keep_first=keep_first, slopes=slopes)
     if max_q is None:
         max_q = int((cu_q[1:] - cu_q[:-1]).max())
     assert q.stride(2) == 1 and out.is_contiguous() and out.shape == (T, H, E) and out.dtype == q.dtype
@@ -198,9 +220,11 @@ def sink_attention_prefill(q, k_cache, v_cache, cu_q, cu_k, block_tables, scale,
         assert gate.stride(1) == 1 and gate.dtype == q.dtype
     _check(_tiles(q.data_ptr(), q.stride(0), q.stride(1), k_cache.data_ptr(), v_cache.data_ptr(),
                   block_tables.data_ptr(), block_tables.stride(0), k_cache.shape[1],
-                  _i32c(cu_q).data_ptr(), _i32(positions).data_ptr(), _f32(sink).data_ptr(),
+                  _i32c(cu_q).data_ptr(), _i32(positions).data_ptr(),
+                  _f32(sink).data_ptr() if sink is not None else None,
                   _ptr(gate), gate.stride(0) if gate is not None else 0, out.data_ptr(), scale,
-                  nseq, 0, max_q, H, G, D, E, _dt(q), _stream()), "sink_attention_prefill")
+                  nseq, 0, max_q, H, G, D, E, int(window), int(keep_first), _slopes(slopes, H),
+                  _dt(q), _stream()), "sink_attention_prefill")
     return out
 
 
@@ -219,7 +243,7 @@ def decode_splits(batch: int, kv_heads: int, heads: int, max_context_len) -> int
 
 
 def sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens, scale, sink, gate, out,
-                          max_context_len=None):
+                          max_context_len=None, window=0, keep_first=0, slopes=None):
     """Single next tokens: row b is sequence b with ``context_lens[b]`` keys.  Head sizes the
     split-context kernel has an instance for (D in 64 / 128 / 256, E in 64 / 128) stream K / V
     rows with coalesced 16-byte loads over several workgroups per sequence and are merged by a
@@ -230,19 +254,24 @@ def sink_attention_decode(q, k_cache, v_cache, block_tables, context_lens, scale
     if (_split_ok(D, E) and q.stride(2) == 1 and q.stride(1) == D and q.data_ptr() % 16 == 0
             and (B == 1 or (q.stride(0) * es) % 16 == 0) and k_cache.is_contiguous()
             and v_cache.is_contiguous() and out.is_contiguous()):
-        splits = decode_splits(B, G, H, max_context_len)
+        seen = max_context_len
+        if window and seen:           # what a row can see bounds the useful splits
+            seen = min(int(seen), int(window) + int(keep_first))
+        splits = decode_splits(B, G, H, seen)
         ws = torch.empty((B * H * splits * (E + 2),), dtype=torch.float32, device=q.device)
         if gate is not None:
             assert gate.stride(1) == 1 and gate.dtype == q.dtype
         _check(_split(q.data_ptr(), q.stride(0) if B > 1 else H * D, q.stride(1), k_cache.data_ptr(),
                       v_cache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0),
-                      k_cache.shape[1], _i32c(context_lens).data_ptr(), _f32(sink).data_ptr(),
+                      k_cache.shape[1], _i32c(context_lens).data_ptr(),
+                      _f32(sink).data_ptr() if sink is not None else None,
                       _ptr(gate), gate.stride(0) if gate is not None else 0, out.data_ptr(),
-                      ws.data_ptr(), scale, B, H, G, D, E, splits, _dt(q), _stream()),
+                      ws.data_ptr(), scale, B, H, G, D, E, splits, int(window), int(keep_first),
+                      _slopes(slopes, H), _dt(q), _stream()),
                "sink_attention_decode")
         return out
     return _attention_rows(q, k_cache, v_cache, block_tables, None, context_lens, 0, scale, sink,
-                           gate, out)
+                           gate, out, 0, window, keep_first, slopes)
 
 
 # ------------------------------------------------------------------ gated delta rule
@@ -253,21 +282,26 @@ def delta_prepare(q, k, v, b, a, conv_w, a_log, dt_bias, conv_state, cu_q, posit
     rs = q.stride(0)
     base = q.data_ptr()
     es = q.element_size()
-    # q, k, v are the first three column blocks of one projection output, b and a views of it
+    # q, k, v are the first three column blocks of one projection output, b a view of it; a is a
+    # view of it too or a tensor of its own, [T, H] (a decay per head) or [T, H*D] (per key channel)
     assert k.data_ptr() == base + G * D * es and v.data_ptr() == base + 2 * G * D * es
-    assert T == 1 or (k.stride(0) == rs and v.stride(0) == rs and b.stride(0) == rs
-                      and a.stride(0) == rs)
-    b_off, a_off = (b.data_ptr() - base) // es, (a.data_ptr() - base) // es
+    assert T == 1 or (k.stride(0) == rs and v.stride(0) == rs and b.stride(0) == rs)
+    assert a.dtype == q.dtype and a.stride(-1) == 1 and a.shape[-1] in (H, H * D)
+    DC = a.shape[-1] // H
+    assert dt_bias.numel() == H * DC
+    b_off = (b.data_ptr() - base) // es
     dev = q.device
     taps = _f32(conv_w).shape[1]
     assert conv_w.shape[0] == 2 * G * D + H * E
     f = dict(dtype=torch.float32, device=dev)
     qn, kn = torch.empty((T, G, D), **f), torch.empty((T, G, D), **f)
-    vv, beta, decay = torch.empty((T, H, E), **f), torch.empty((T, H), **f), torch.empty((T, H), **f)
+    vv, beta = torch.empty((T, H, E), **f), torch.empty((T, H), **f)
+    decay = torch.empty((T, H) if DC == 1 else (T, H, D), **f)
     if cu_q is not None:
         assert row_seq is not None, "prefill-form steps pass the sequence of each row"
     B = slots.shape[0]
-    _check(_prep(base, rs, b_off, a_off, conv_w.data_ptr(), taps, _f32(a_log).data_ptr(),
+    _check(_prep(base, rs if T > 1 else int(rs or 0), b_off, a.data_ptr(), a.stride(0), DC,
+                 conv_w.data_ptr(), taps, _f32(a_log).data_ptr(),
                  _f32(dt_bias).data_ptr(), _f32(conv_state).data_ptr(), _ptr(_i32(cu_q)),
                  _i32(positions).data_ptr(), _i32(slots).data_ptr(),
                  _ptr(_i32(row_seq)) if cu_q is not None else None, qn.data_ptr(), kn.data_ptr(),
@@ -281,6 +315,13 @@ def delta_scan(qn, kn, vv, beta, decay, state, cu_q, positions, slots):
     H, E = vv.shape[1], vv.shape[2]
     assert state.shape[1:] == (H, D, E)
     o = torch.zeros((T, H, E), dtype=torch.float32, device=qn.device)
+    if decay.dim() == 3:                 # a decay per head and key channel
+        assert decay.shape == (T, H, D) and decay.is_contiguous()
+        _check(_cscan(qn.data_ptr(), kn.data_ptr(), vv.data_ptr(), beta.data_ptr(), decay.data_ptr(),
+                      _f32(state).data_ptr(), _ptr(_i32(cu_q)), _i32(positions).data_ptr(),
+                      _i32(slots).data_ptr(), o.data_ptr(), slots.shape[0], H, G, D, E, _stream()),
+               "channel_delta_scan")
+        return o
     _check(_scan(qn.data_ptr(), kn.data_ptr(), vv.data_ptr(), beta.data_ptr(), decay.data_ptr(),
                  _f32(state).data_ptr(), _ptr(_i32(cu_q)), _i32(positions).data_ptr(),
                  _i32(slots).data_ptr(), o.data_ptr(), slots.shape[0], H, G, D, E, _stream()),
@@ -288,23 +329,26 @@ def delta_scan(qn, kn, vv, beta, decay, state, cu_q, positions, slots):
     return o
 
 
-def gated_head_norm(o, w, gate, eps, out_dtype):
+def gated_head_norm(o, w, gate, eps, out_dtype, act="silu"):
     T, H, E = o.shape
-    assert gate.stride(-1) == 1 and gate.dtype == out_dtype
+    assert gate.stride(-1) == 1 and gate.dtype == out_dtype and w.numel() in (E, H * E)
+    assert act in ("silu", "sigmoid")
     out = torch.empty((T, H, E), dtype=out_dtype, device=o.device)
     _check(_ghn(_f32(o).data_ptr(), _f32(w).data_ptr(), gate.data_ptr(), gate.stride(0),
-                out.data_ptr(), T, H, E, eps, _dt(out), _stream()), "gated_head_norm")
+                out.data_ptr(), T, H, E, eps, int(w.numel() == H * E and H > 1), int(act == "sigmoid"),
+                _dt(out), _stream()), "gated_head_norm")
     return out
 
 
 # ------------------------------------------------------------------ grouped expert routing
-def grouped_route(h, router_w, top, groups, keep):
+def grouped_route(h, router_w, top, groups, keep, score="softmax"):
+    assert score in ("softmax", "sigmoid")
     T, W = h.shape
     NE = router_w.shape[0]
     assert h.is_contiguous()
     dense = torch.empty((T, NE), dtype=torch.float32, device=h.device)
     _check(_route(h.data_ptr(), _f32(router_w).data_ptr(), dense.data_ptr(), T, W, NE, top, groups,
-                  keep, _dt(h), _stream()), "grouped_route")
+                  keep, int(score == "sigmoid"), _dt(h), _stream()), "grouped_route")
     return dense
 
 
@@ -316,3 +360,118 @@ def gelu_route_scale(up, dense, ff, out_dtype):
     _check(_gelu(up.data_ptr(), _f32(dense).data_ptr(), act.data_ptr(), T, NE, ff, _dt(up),
                  _stream()), "gelu_route_scale")
     return act
+
+
+def swiglu_route_scale(gu, dense, ff, shared_ff, out_dtype):
+    T = gu.shape[0]
+    C = gu.shape[1] // 2
+    NE = dense.shape[1] if dense is not None else 0
+    assert gu.stride(1) == 1 and gu.dtype == out_dtype and C == NE * ff + shared_ff
+    act = torch.empty((T, C), dtype=out_dtype, device=gu.device)
+    _check(_swi(gu.data_ptr(), _rows(gu), _ptr(_f32(dense)) if dense is not None else None,
+                act.data_ptr(), T, NE, ff if NE else 1, shared_ff, _dt(gu), _stream()),
+           "swiglu_route_scale")
+    return act
+
+
+# ------------------------------------------------------------------ positions, grouped norms
+def embed_sinusoid(ids, positions, table, inv_freq):
+    T, W = ids.shape[0], table.shape[1]
+    assert table.is_contiguous() and inv_freq.numel() == W // 2
+    x = torch.empty((T, W), dtype=torch.float32, device=table.device)
+    _check(_esin(_i32(ids).data_ptr(), _i32(positions).data_ptr(), table.data_ptr(),
+                 _f32(inv_freq).data_ptr(), x.data_ptr(), T, W, _dt(table), _stream()), "embed_sinusoid")
+    return x
+
+
+def group_rms_norm(x, w, groups, eps, out_dtype):
+    return residual_group_norm(x, (), w, groups, eps, out_dtype)
+
+
+def residual_group_norm(x, ys, w_next, groups, eps, out_dtype):
+    x = _f32(x)
+    T, W = x.shape
+    ys = list(ys)
+    assert len(ys) <= 2, "at most two branches are added per call"
+    for y in ys:
+        assert y.shape == x.shape and y.stride(1) == 1 and y.dtype == out_dtype
+    h = torch.empty((T, W), dtype=out_dtype, device=x.device) if w_next is not None else None
+    if h is None and not ys:
+        return None
+    y1 = ys[0] if ys else None
+    y2 = ys[1] if len(ys) > 1 else None
+    _check(_rgn(x.data_ptr(), _ptr(y1), _rows(y1) if y1 is not None else 0, _ptr(y2),
+                _rows(y2) if y2 is not None else 0, _ptr(w_next), _ptr(h), T, W, groups, eps,
+                _DT[out_dtype], _stream()), "residual_group_norm")
+    return h
+
+
+def add_normed_mean(x, parts, eps):
+    x = _f32(x)
+    T, W = x.shape
+    assert 1 <= len(parts) <= 2
+    (y1, w1), (y2, w2) = parts[0], (parts[1] if len(parts) > 1 else (None, None))
+    for y in (y1, y2):
+        assert y is None or (y.shape == x.shape and y.stride(1) == 1 and y.dtype == y1.dtype)
+    _check(_anm(x.data_ptr(), y1.data_ptr(), _rows(y1), _f32(w1).data_ptr(), _ptr(y2),
+                _rows(y2) if y2 is not None else 0, _f32(w2).data_ptr() if w2 is not None else None,
+                T, W, eps, _dt(y1), _stream()), "add_normed_mean")
+
+
+def unit_norm_store(q, k, eps, k_cache, v_cache, slot_mapping):
+    T, H, D = q.shape
+    G = k.shape[1]
+    rs = q.stride(0)
+    assert (T == 1 or k.stride(0) == rs) and q.stride(1) == D and k.stride(1) == D \
+        and q.stride(2) == 1 and k.stride(2) == 1, "q / k must be views of one projection output"
+    if k_cache is not None:
+        assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dtype == q.dtype \
+            and k_cache.shape[2:] == (G, D) and v_cache.shape[2:] == (G, D)
+    _check(_uns(q.data_ptr(), k.data_ptr(), rs, eps, _ptr(k_cache), _ptr(v_cache),
+                _ptr(_i32(slot_mapping)), T, H, G, D, _dt(q), _stream()), "unit_norm_store")
+
+
+def tanh_cap_(z, cap):
+    assert z.is_contiguous()
+    _check(_cap(z.data_ptr(), z.numel(), cap, _dt(z), _stream()), "tanh_cap")
+    return z
+
+
+# ------------------------------------------------------------------ gated outer-product recurrences
+def _heads_view(t, n):
+    """Element stride per token of a [T, heads, n] view whose heads are dense."""
+    assert t.stride(2) == 1 and t.stride(1) == n
+    return _rows(t)
+
+
+def mlstm_scan(q, k, v, i_raw, f_raw, i_bias, f_bias, cap, state, norm_state, max_state,
+               cu_q, positions, slots):
+    T, H, D = q.shape
+    E = v.shape[2]
+    assert state.shape[1:] == (H, D, E) and norm_state.shape[1:] == (H, D) and max_state.shape[1:] == (H,)
+    assert i_raw.shape == (T, H) and f_raw.shape == (T, H) and i_raw.stride(1) == 1 and f_raw.stride(1) == 1
+    assert T == 1 or i_raw.stride(0) == f_raw.stride(0)
+    assert k.dtype == q.dtype and v.dtype == q.dtype and i_raw.dtype == q.dtype and f_raw.dtype == q.dtype
+    o = torch.zeros((T, H, E), dtype=torch.float32, device=q.device)
+    _check(_mlstm(q.data_ptr(), k.data_ptr(), v.data_ptr(), _heads_view(q, D), _heads_view(k, D),
+                  _heads_view(v, E), i_raw.data_ptr(), f_raw.data_ptr(), _rows(i_raw),
+                  _f32(i_bias).data_ptr(), _f32(f_bias).data_ptr(), cap, _f32(state).data_ptr(),
+                  _f32(norm_state).data_ptr(), _f32(max_state).data_ptr(), _ptr(_i32(cu_q)),
+                  _i32(positions).data_ptr(), _i32(slots).data_ptr(), o.data_ptr(), slots.shape[0],
+                  H, D, E, _dt(q), _stream()), "mlstm_scan")
+    return o
+
+
+def gla_scan(q, k, v, a_raw, a_bias, tau, state, cu_q, positions, slots):
+    T, H, D = q.shape
+    E = v.shape[2]
+    assert state.shape[1:] == (H, D, E) and a_raw.shape == (T, H * D) and a_raw.stride(1) == 1
+    assert k.dtype == q.dtype and v.dtype == q.dtype and a_raw.dtype == q.dtype
+    assert a_bias.numel() == H * D
+    o = torch.zeros((T, H, E), dtype=torch.float32, device=q.device)
+    _check(_gla(q.data_ptr(), k.data_ptr(), v.data_ptr(), _heads_view(q, D), _heads_view(k, D),
+                _heads_view(v, E), a_raw.data_ptr(), _rows(a_raw), _f32(a_bias).data_ptr(), tau,
+                _f32(state).data_ptr(), _ptr(_i32(cu_q)), _i32(positions).data_ptr(),
+                _i32(slots).data_ptr(), o.data_ptr(), slots.shape[0], H, D, E, _dt(q), _stream()),
+           "gla_scan")
+    return o
