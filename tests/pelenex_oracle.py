@@ -162,14 +162,19 @@ def gated_ff(x, p):
     return lin(p["down"], silu(lin(p["gate"], x)) * lin(p["up"], x))
 
 
-def feed_forward(h, p, f):
+def feed_forward(h, p, f, margins=None):
+    """``margins`` (a list of length T): lowered to the gap between the last chosen and the best
+    rejected score of every token (how close the routing decision is)."""
     if f["kind"] == "dense":
         return gated_ff(h, p)
     n, top = f["router"]["experts"], f["router"]["top"]
     s = torch.sigmoid(lin(p["router"], h))
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
-        order = sorted(range(n), key=lambda e: (-float(s[t, e]), e))[:top]
+        ranked = sorted(range(n), key=lambda e: (-float(s[t, e]), e))
+        order = ranked[:top]
+        if margins is not None and top < n:
+            margins[t] = min(margins[t], float(s[t, ranked[top - 1]] - s[t, ranked[top]]))
         for e in order:
             pe = {k[len(f"e{e}."):]: v for k, v in p.items() if k.startswith(f"e{e}.")}
             out[t] += gated_ff(s[t, e] * h[t], pe)
@@ -182,8 +187,9 @@ def feed_forward(h, p, f):
 MIXERS = {"mlstm": mlstm, "parallel": parallel_mixer, "channel_delta": channel_delta}
 
 
-def forward(cfg: dict, ckpt: dict, tokens):
-    """Returns (logits [T, vocab], stream after every layer [layers, T, W]), float64."""
+def forward(cfg: dict, ckpt: dict, tokens, margins=None):
+    """Returns (logits [T, vocab], stream after every layer [layers, T, W]), float64.  ``margins``:
+    see ``feed_forward``."""
     W, eps, groups = cfg["width"], float(cfg["norm"]["eps"]), cfg["norm"]["groups"]
     T = len(tokens)
     x = ckpt["embed"].to(F64)[torch.tensor(tokens)] + torch.stack([sinusoid(t, W) for t in range(T)])
@@ -195,7 +201,8 @@ def forward(cfg: dict, ckpt: dict, tokens):
         y = MIXERS[L["type"]](h, {k[4:]: v for k, v in p.items() if k.startswith("mix.")},
                               L["mixer"], eps)
         if L.get("mlp"):
-            y = y + feed_forward(h, {k[4:]: v for k, v in p.items() if k.startswith("mlp.")}, L["mlp"])
+            y = y + feed_forward(h, {k[4:]: v for k, v in p.items() if k.startswith("mlp.")}, L["mlp"],
+                                 margins)
         x = x + y
         streams.append(x.clone())
     z = lin(ckpt["head"], group_norm(x, ckpt["final.norm"], groups, eps))

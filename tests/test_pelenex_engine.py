@@ -1,0 +1,373 @@
+"""The Pelenex family inside the engine (registry, loader, scheduler, paged KV + state slots,
+kernels) against the plain oracle of ``pelenex_oracle``: every mixer and feed-forward kind alone
+(one-layer models), whole prompts and the stream after every layer, token-by-token decoding,
+portions down to two tokens, mixed batches against each request alone, blocks and slots that are
+used again, keys that stand out far back / at block borders / just inside and outside the window
+and the kept first tokens (in prompts and while decoding), long decoding, sizes that are 1 or
+equal, greedy generation through ``LLMEngine.generate``, and the replay entry point.  Every test
+runs on the CPU (fp32); the ``gpu`` variants run the HIP kernels in float32 and bfloat16."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import pelenex_fixtures as fx
+import pelenex_oracle as oracle
+
+from minivllm_amd.engine.llm_engine import LLMEngine
+from minivllm_amd.models.registry import config_from_path
+from minivllm_amd.sampling_parameters import SamplingParams
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CASES = [pytest.param("cpu", "float32", id="cpu-fp32"),
+         pytest.param("cuda", "float32", id="gpu-fp32", marks=pytest.mark.gpu),
+         pytest.param("cuda", "bfloat16", id="gpu-bf16", marks=pytest.mark.gpu)]
+
+
+def make_engine(tmp_path, c, w, device, dtype, blocks=24, block_size=8, seqs=3, score=True, **kw):
+    folder = fx.save_checkpoint(str(tmp_path / "ckpt"), c, w)
+    mc = config_from_path(folder)
+    assert type(mc).__name__ == "PelenexConfig"
+    cfg = dict(model=mc, checkpoint_path=folder, dtype=dtype, device=device,
+               block_size=block_size, max_cached_blocks=blocks, max_num_sequences=seqs,
+               max_model_length=blocks * block_size,
+               max_num_batched_tokens=blocks * block_size, eos=-1, score_only=score,
+               graph_batch_sizes=[1, 2, seqs], tuned_gemms=False)
+    cfg.update(kw)
+    return LLMEngine(cfg)
+
+
+def tokens(n, vocab, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+class Expected:
+    """The oracle's logits and streams for a token list, and the first token at which one of its
+    routing decisions is a close call (16-bit rounding may decide it the other way, and the
+    recurrent state then carries the difference on): bfloat16 runs are compared up to there."""
+
+    def __init__(self, c, w, toks):
+        margins = [1.0] * len(toks)
+        self.logits, self.trace = oracle.forward(c, w, toks, margins)
+        close_calls = [t for t, m in enumerate(margins) if m < 0.05]
+        self.sure = close_calls[0] if close_calls else len(toks)
+
+
+def close(got, want, dtype):
+    """Error of a logit row: spread of the difference over the vocabulary relative to the spread
+    of the logits themselves."""
+    n = want.logits.shape[0] if dtype == "float32" else want.sure
+    if n == 0:
+        return
+    d = got[:n].double() - want.logits[:n]
+    d = d - d.mean(-1, keepdim=True)
+    e = d.pow(2).mean(-1).sqrt() / want.logits[:n].std(-1)
+    lim = 2e-4 if dtype == "float32" else 0.25
+    assert float(e.max()) < lim, f"logits differ: {float(e.max()):.3g} at {int(e.argmax())} (limit {lim})"
+    if dtype != "float32":
+        assert float(e.median()) < 0.05, f"typical row differs: {float(e.median()):.3g}"
+
+
+def run_schedule(eng, reqs, schedule):
+    """``schedule``: list of steps, each a list of (name, count).  Returns name -> [len, V]."""
+    at = {k: 0 for k in reqs}
+    got = {k: [] for k in reqs}
+    for step in schedule:
+        entries, end = [], []
+        for name, n in step:
+            lo = at[name]
+            entries.append({"id": name, "tokens": reqs[name][lo:lo + n], "want": list(range(n))})
+            at[name] = lo + n
+            if at[name] == len(reqs[name]):
+                end.append(name)
+        out = eng.score_step(entries, end)
+        for name, _ in step:
+            got[name].append(out[name])
+    return {k: torch.cat(v) for k, v in got.items() if v}
+
+
+ALONE = {
+    "mlstm": [(fx.mlstm(), None)],
+    "mlstm-capped-gates": [(fx.mlstm(heads=2, dim=20, vdim=12, cap=1.5), None)],
+    "parallel": [(fx.parallel(), None)],
+    "delta": [(fx.delta(), None)],
+    "delta-one-tap-shared-qk": [(fx.delta(heads=6, kv_heads=1, dim=8, vdim=12, conv=1), None)],
+    "dense-ff": [(fx.mlstm(heads=1, dim=8, vdim=8), fx.dense())],
+    "moe-top1": [(fx.mlstm(heads=1, dim=8, vdim=8), fx.moe(top=1))],
+    "moe-all-no-shared": [(fx.mlstm(heads=1, dim=8, vdim=8), fx.moe(experts=3, top=3, shared=0))],
+    "moe-one-expert": [(fx.mlstm(heads=1, dim=8, vdim=8), fx.moe(experts=1, top=1, shared=24))],
+}
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+@pytest.mark.parametrize("kind", list(ALONE))
+def test_each_mechanism_alone(tmp_path, device, dtype, kind):
+    """One-layer models: whole prompt, then the same tokens as a prompt portion + single tokens."""
+    c = fx.config(ALONE[kind], width=32, vocab=53, groups=2)
+    w = fx.weights(c, 40)
+    toks = tokens(33, c["vocab"], 41)
+    eng = make_engine(tmp_path, c, w, device, dtype)
+    seen = []
+    eng.model_runner.model.model.layer_hook = lambda i, x: seen.append(x.detach().float().cpu().clone())
+    want = Expected(c, w, toks)
+    close(run_schedule(eng, {"a": toks}, [[("a", len(toks))]])["a"], want, dtype)
+    n = len(toks) if dtype == "float32" else want.sure
+    lim = 1e-4 if dtype == "float32" else 0.1
+    assert float((seen[0][:n].double() - want.trace[0][:n]).abs().max()) < lim * float(want.trace[0].abs().max())
+    eng.model_runner.model.model.layer_hook = None
+    close(run_schedule(eng, {"b": toks}, [[("b", 5)], [("b", 17)]] + [[("b", 1)]] * 11)["b"], want, dtype)
+    eng.exit()
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_whole_prompt_and_every_layer(tmp_path, device, dtype):
+    c = fx.default_config()
+    w = fx.weights(c, 1)
+    toks = tokens(37, c["vocab"], 2)
+    eng = make_engine(tmp_path, c, w, device, dtype)
+    seen = []
+    eng.model_runner.model.model.layer_hook = lambda i, x: seen.append(x.detach().float().cpu().clone())
+    got = run_schedule(eng, {"a": toks}, [[("a", len(toks))]])["a"]
+    want = Expected(c, w, toks)
+    close(got, want, dtype)
+    assert len(seen) == len(c["layers"])
+    n = len(toks) if dtype == "float32" else want.sure
+    assert n >= 8, "the fixture's routing is a close call too early for a 16-bit comparison"
+    for x, ref in zip(seen, want.trace):
+        lim = 1e-4 if dtype == "float32" else 0.15
+        assert float((x[:n].double() - ref[:n]).abs().max()) < lim * float(ref.abs().max())
+    eng.exit()
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_token_by_token_equals_prefill(tmp_path, device, dtype):
+    c = fx.default_config()
+    w = fx.weights(c, 3)
+    toks = tokens(29, c["vocab"], 4)
+    eng = make_engine(tmp_path, c, w, device, dtype)
+    want = Expected(c, w, toks)
+    close(run_schedule(eng, {"a": toks}, [[("a", 1)] for _ in toks])["a"], want, dtype)   # first tokens, then decode
+    close(run_schedule(eng, {"b": toks}, [[("b", 20)]] + [[("b", 1)]] * 9)["b"], want, dtype)
+    eng.exit()
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+@pytest.mark.parametrize("cuts", [[2, 2, 3, 1, 9, 8, 2, 16, 2, 5], [7, 43], [1, 2, 47], [25, 25]])
+def test_portions_cut_anywhere(tmp_path, device, dtype, cuts):
+    c = fx.default_config()
+    w = fx.weights(c, 5)
+    toks = tokens(sum(cuts), c["vocab"], 6)
+    eng = make_engine(tmp_path, c, w, device, dtype)
+    got = run_schedule(eng, {"a": toks}, [[("a", n)] for n in cuts])["a"]
+    close(got, Expected(c, w, toks), dtype)
+    eng.exit()
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_mixed_batches_equal_each_request_alone(tmp_path, device, dtype):
+    c = fx.default_config()
+    w = fx.weights(c, 7)
+    reqs = {"a": tokens(41, c["vocab"], 8), "b": tokens(5, c["vocab"], 9), "c": tokens(23, c["vocab"], 10),
+            "d": tokens(1, c["vocab"], 11), "e": tokens(18, c["vocab"], 12)}
+    sched = [[("a", 9), ("b", 2)],
+             [("a", 1), ("b", 1), ("c", 17)],              # a one-token portion next to a prompt
+             [("b", 1), ("c", 1)],                         # decode step of two; a sits out
+             [("a", 20), ("b", 1), ("c", 1)],              # b ends: its slot and blocks return
+             [("a", 1), ("c", 1), ("d", 1)],               # d takes b's slot, first token alone
+             [("e", 3), ("a", 1), ("c", 1)],
+             [("e", 15), ("a", 9), ("c", 2)]]
+    eng = make_engine(tmp_path, c, w, device, dtype, blocks=14, seqs=3)
+    got = run_schedule(eng, reqs, sched)
+    for k, toks in reqs.items():
+        close(got[k], Expected(c, w, toks), dtype)
+    bm = eng.scheduler.block_manager
+    assert bm.num_free_blocks == bm.num_blocks and eng.scheduler.state_pool.num_free == 3
+    eng.exit()
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_pool_and_slots_used_again(tmp_path, device, dtype):
+    """Two slots, a KV pool of just over one request: every later request runs on blocks and a
+    slot (matrix state, normaliser, running maximum, convolution tail) that an earlier one has
+    left dirty."""
+    c = fx.default_config()
+    w = fx.weights(c, 13)
+    eng = make_engine(tmp_path, c, w, device, dtype, blocks=9, seqs=2)
+    for i, n in enumerate([60, 33, 64, 9, 2]):
+        toks = tokens(n, c["vocab"], 20 + i)
+        cut = max(1, n // 3)
+        got = run_schedule(eng, {"r": toks}, [[("r", cut)], [("r", n - cut)]] if n > 1 else [[("r", 1)]])["r"]
+        close(got, Expected(c, w, toks), dtype)
+    eng.exit()
+
+
+def _standout_model(size, keep, bs):
+    """One parallel layer made so that ONE key stands out for the last query: the embedding is
+    larger than the position vector, the attention branch has a large output weight, token 38's row is token 39's with its halves swapped, and
+    the key projection is the second query head's with its input columns swapped the same way, so
+    k(token 38) = q_1(token 39) - the largest score a unit q and k can have - wherever token 38
+    sits, while its value (the key before the norm) is unlike every other token's."""
+    W = 32
+    c = fx.config([(fx.parallel(heads=2, kv_heads=1, dim=16, size=size, keep=keep, scale=1.5,
+                                rheads=1, rdim=8, rvdim=8), None)], width=W, vocab=40, groups=1)
+    w = fx.weights(c, 50)
+    q1 = w["l0.mix.left.q"][16:32]                                # head 1: the smaller distance penalty
+    w["l0.mix.left.k"] = torch.cat([q1[:, W // 2:], q1[:, :W // 2]], 1).contiguous()
+    w["l0.norm1"] = torch.ones(W, dtype=torch.bfloat16)
+    w["l0.mix.left.out"] = torch.full((W,), 4.0, dtype=torch.bfloat16)
+    e = (w["embed"].float() * 6).to(torch.bfloat16)
+    e[38] = torch.cat([e[39, W // 2:], e[39, :W // 2]])
+    w["embed"] = e
+    return c, w
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+@pytest.mark.parametrize("decoded", [False, True], ids=["prompt", "decoded"])
+def test_keys_at_every_edge(tmp_path, device, dtype, decoded):
+    """Token 38 sits at a key position, token 39 at the query position (the last one); key
+    positions: the very first token, the last kept one and the first not kept, both sides of a
+    block border, far back but kept, just inside and just outside the window.  The oracle's logits
+    for a key on either side of an edge differ widely, so a window or a kept prefix that is off by
+    one cannot pass."""
+    size, keep, bs, n = 11, 4, 8, 41
+    c, w = _standout_model(size, keep, bs)
+    q = n - 1
+    places = [0, keep - 1, keep, bs - 1, bs, 2 * bs - 1, q - size + 1, q - size, q - 1]
+    eng = make_engine(tmp_path, c, w, device, dtype, blocks=12, block_size=bs, seqs=2)
+    seen_logits = {}
+    for j in places:
+        toks = [1 + (t * 7) % 37 for t in range(n)]            # ids 1 .. 37
+        toks[j], toks[q] = 38, 39
+        sched = [[("a", n)]] if not decoded else [[("a", n - 6)]] + [[("a", 1)]] * 6
+        got = run_schedule(eng, {"a": toks}, sched)["a"]
+        want = Expected(c, w, toks)
+        close(got, want, dtype)
+        seen_logits[j] = want.logits[q]
+    spread = float(seen_logits[0].std())
+    for inside, outside in ((keep - 1, keep), (q - size + 1, q - size)):
+        assert float((seen_logits[inside] - seen_logits[outside]).std()) > 0.1 * spread, \
+            "the fixture does not tell a visible key from a hidden one"
+    eng.exit()
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_long_decoding_over_many_blocks(tmp_path, device, dtype):
+    """150 single tokens: the window and the kept first tokens pass over decoded tokens and many
+    block borders, the recurrent states run long."""
+    c = fx.config([(fx.parallel(heads=2, kv_heads=2, dim=8, size=21, keep=2, rheads=1, rdim=8, rvdim=4), None),
+                   (fx.mlstm(heads=2, dim=8, vdim=4, cap=4.0), fx.moe(experts=4, top=4, shared=0)),
+                   (fx.delta(heads=1, kv_heads=1, dim=16, vdim=4, conv=4), None)],
+                  width=24, vocab=61, groups=3)
+    w = fx.weights(c, 14)
+    toks = tokens(150, c["vocab"], 15)
+    eng = make_engine(tmp_path, c, w, device, dtype, blocks=40, block_size=4)
+    got = run_schedule(eng, {"a": toks}, [[("a", 3)]] + [[("a", 1)]] * 147)["a"]
+    close(got, Expected(c, w, toks), dtype)
+    eng.exit()
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_sizes_that_happen_to_be_one_or_equal(tmp_path, device, dtype):
+    """One head, one norm group, one expert, top = every expert, taps = 1, heads == kv heads, no
+    kept tokens, a window longer than the text, no soft cap, key size != value size."""
+    for layers, kw in (([(fx.parallel(heads=1, kv_heads=1, dim=8, size=100, keep=0, rheads=1, rdim=8, rvdim=8),
+                          fx.moe(experts=2, top=2, shared=8))], dict(groups=1, softcap=0.0)),
+                       ([(fx.delta(heads=1, kv_heads=1, dim=8, vdim=8, conv=1), None)], dict(groups=16)),
+                       ([(fx.mlstm(heads=5, dim=4, vdim=36), fx.dense(8)),
+                         (fx.parallel(heads=8, kv_heads=1, dim=6, size=1, keep=30, rheads=3, rdim=70, rvdim=2), None),
+                         (fx.delta(heads=6, kv_heads=3, dim=4, vdim=36, conv=6), fx.moe(experts=8, top=3))],
+                        dict(groups=8))):
+        c = fx.config(layers, width=16, vocab=50, **kw)
+        w = fx.weights(c, 16)
+        toks = tokens(21, c["vocab"], 17)
+        eng = make_engine(tmp_path, c, w, device, dtype)
+        got = run_schedule(eng, {"a": toks}, [[("a", 2)], [("a", 12)]] + [[("a", 1)]] * 7)["a"]
+        close(got, Expected(c, w, toks), dtype)
+        eng.exit()
+
+
+def _follow(c, w, prompt, gen, dtype):
+    """Greedy tokens against the oracle (recomputed from scratch per token: it keeps no state)."""
+    toks = list(prompt)
+    for t in gen:
+        lg = oracle.forward(c, w, toks)[0][-1]
+        top2 = lg.topk(2).values
+        if dtype == "bfloat16" and float(top2[0] - top2[1]) < 0.15:
+            break                          # a near tie: 16-bit rounding may pick either
+        assert int(lg.argmax()) == t
+        toks.append(t)
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_greedy_generation_through_the_scheduler(tmp_path, device, dtype):
+    c = fx.default_config()
+    w = fx.weights(c, 18)
+    prompts = [tokens(n, c["vocab"], 30 + n) for n in (11, 3, 26, 1)]
+    eng = make_engine(tmp_path, c, w, device, dtype, score=False, seqs=3, blocks=30,
+                      max_num_batched_tokens=32)
+    out = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True))
+    for p, gen in zip(prompts, out["token_ids"]):
+        assert len(gen) == 8
+        _follow(c, w, p, gen, dtype)
+    eng.exit()
+
+
+@pytest.mark.parametrize("device,dtype", CASES[:2])
+def test_generation_survives_preemption_and_mixed_steps(tmp_path, device, dtype):
+    c = fx.default_config()
+    w = fx.weights(c, 19)
+    prompts = [tokens(n, c["vocab"], 60 + n) for n in (21, 17, 9, 30)]
+    eng = make_engine(tmp_path, c, w, device, dtype, score=False, seqs=3, blocks=11, block_size=8,
+                      max_num_batched_tokens=24, enable_mixed_batches=True)
+    out = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=14, ignore_eos=True))
+    assert eng.scheduler.num_preemptions > 0 and eng.scheduler.num_mixed_steps > 0
+    for p, gen in zip(prompts, out["token_ids"]):
+        _follow(c, w, p, gen, dtype)
+    assert eng.scheduler.state_pool.num_free == 3
+    eng.exit()
+
+
+def test_replay_entry_point_writes_the_oracles_logits(tmp_path):
+    c = fx.default_config()
+    w = fx.weights(c, 21)
+    folder = fx.save_checkpoint(str(tmp_path / "m"), c, w)
+    a, b = tokens(70, c["vocab"], 22), tokens(9, c["vocab"], 23)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:40], "want": [0, 39]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[40:69], "want": []},
+                                     {"id": "b", "tokens": b[:8], "want": [7]}], "end": []},
+             {"step": 2, "entries": [{"id": "b", "tokens": b[8:], "want": [0]},
+                                     {"id": "a", "tokens": a[69:], "want": [0]}], "end": ["a", "b"]}]
+    out = tmp_path / "out"
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder,
+                        "--dtype", "float32", "--out", str(out), "--max-tokens", "192",
+                        "--block-size", "16", "--device", "cpu"],
+                       input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True,
+                       text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [l for l in p.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    la, lb = oracle.forward(c, w, a)[0].float().numpy(), oracle.forward(c, w, b)[0].float().numpy()
+    V = c["vocab"]
+    got = {n: np.fromfile(out / f"{n}.f32", "<f4").reshape(-1, V) for n in range(3)}
+    np.testing.assert_allclose(got[0], la[[0, 39]], rtol=2e-4, atol=2e-4)
+    np.testing.assert_allclose(got[1], lb[[7]], rtol=2e-4, atol=2e-4)
+    np.testing.assert_allclose(got[2], np.stack([lb[8], la[69]]), rtol=2e-4, atol=2e-4)
+
+
+def test_checkpoint_errors_name_the_tensor(tmp_path):
+    c = fx.config(ALONE["delta"], width=32, vocab=53)
+    w = fx.weights(c, 60)
+    bad = dict(w)
+    del bad["l0.mix.a2"]
+    with pytest.raises(KeyError, match="l0.mix.a2"):
+        make_engine(tmp_path / "x", c, bad, "cpu", "float32")
+    bad = dict(w, **{"l0.mix.extra": torch.zeros(3)})
+    with pytest.raises(KeyError, match="l0.mix.extra"):
+        make_engine(tmp_path / "y", c, bad, "cpu", "float32")
+    bad = dict(w, **{"l0.mix.q": torch.zeros(7, 32)})
+    with pytest.raises(ValueError, match="l0.mix.q"):
+        make_engine(tmp_path / "z", c, bad, "cpu", "float32")
