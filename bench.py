@@ -309,9 +309,37 @@ def hybrid_models(size: str, vocab: int = 32768, experts: int = 4, top: int = 2)
     return hybrid, dense
 
 
+def pelenex_model(size: str, vocab: int = 32768, experts: int = 4, top: int = 2, window: int = 512):
+    """Pelenex configuration of the same width, depth, head geometry and active feed-forward
+    parameters per token as ``hybrid_models(size)``: layers cycle through matrix LSTM, the
+    parallel mixer (windowed attention + gated linear attention), channel-decay delta rule and
+    the parallel mixer again; every layer has routed gated experts plus a shared one
+    ((top + 1) * 3 * ff = 3 * intermediate)."""
+    from minivllm_amd.models.pelenex import PelenexConfig
+    W, L, H, G, D, inter = HYBRID_SIZES[size]
+    ff = inter // (top + 1) // 64 * 64
+    mlp = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top},
+           "shared": {"ff": ff}}
+    kinds = [("mlstm", {"heads": H // 2, "dim": D, "vdim": D, "gate_cap": 15.0}),
+             ("parallel", {"left": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5 * 4,
+                                    "mask": {"size": window, "keep_first": 4}},
+                           "right": {"heads": H // 2, "dim": D // 2, "vdim": D, "tau": 16.0}}),
+             ("channel_delta", {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "conv": 4})]
+    order = [0, 1, 2, 1]
+    layers = [{"type": kinds[order[i % 4]][0], "mixer": kinds[order[i % 4]][1], "mlp": mlp}
+              for i in range(L)]
+    return PelenexConfig.from_dict({"architecture": "Pelenex", "vocab": vocab, "width": W,
+                                    "norm": {"eps": 1e-6, "groups": 4}, "logit_softcap": 30.0,
+                                    "layers": layers, "max_position": 8192}, name=f"pelenex-{size}")
+
+
 def hybrid_comparison(args) -> dict:
-    """Prefill and decode throughput of the hybrid family next to the dense decoder of the same
-    size, one GPU, same engine path as the headline measurement (``bench_model``)."""
+    """Prefill and decode throughput of the hybrid families next to the dense decoder of the same
+    size, one GPU, same engine path as the headline measurement (``bench_model``).
+    ``--family natilix`` (default): Natilix and dense; ``--family pelenex``: Pelenex, Natilix (its
+    closest relative: attention + delta rule + routed experts around a fp32 stream) and dense."""
+    if args.family == "pelenex":
+        return pelenex_comparison(args)
     out = {"metric": "prefill / decode tok/s, hybrid (attention + delta rule + routed experts) "
                      "next to the dense decoder of equal size",
            "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -330,6 +358,31 @@ def hybrid_comparison(args) -> dict:
         for k in ("prefill_tok_s", "decode_tok_s"):
             if k in row["hybrid"] and k in row["dense"]:
                 row[f"hybrid_over_dense_{k}"] = round(row["hybrid"][k] / row["dense"][k], 3)
+        out["sizes"][size] = row
+    return out
+
+
+def pelenex_comparison(args) -> dict:
+    out = {"metric": "prefill / decode tok/s, Pelenex (matrix LSTM, windowed attention + gated "
+                     "linear attention, channel-decay delta rule, routed gated experts) next to "
+                     "Natilix and the dense decoder of equal size",
+           "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "dtype": "bf16", "data": "synthetic random token prompts, random-init weights",
+           "config": {"seq_len": args.seq_len, "decode_batch": args.batch,
+                      "prefill_tokens_per_step": args.prefill_tokens, "kv_block_size": args.block_size},
+           "sizes": {}}
+    keep = ("prefill_tok_s", "prefill_ms_per_step", "decode_tok_s", "decode_ms_per_step",
+            "hipgraph_captured", "init_s")
+    for size in args.hybrid.split(","):
+        natilix, dense = hybrid_models(size)
+        row = {}
+        for name, model in (("pelenex", pelenex_model(size)), ("natilix", natilix), ("dense", dense)):
+            r = bench_model(args, model, 0, 1)
+            row[name] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in r.items() if k in keep}
+        for k in ("prefill_tok_s", "decode_tok_s"):
+            if all(k in row[n] for n in ("pelenex", "natilix", "dense")):
+                row[f"pelenex_over_natilix_{k}"] = round(row["pelenex"][k] / row["natilix"][k], 3)
+                row[f"pelenex_over_dense_{k}"] = round(row["pelenex"][k] / row["dense"][k], 3)
         out["sizes"][size] = row
     return out
 
@@ -633,6 +686,9 @@ def main():
                          "launch floor of a real N-GPU run; NOT a scaling number)")
     ap.add_argument("--p2p", action="store_true",
                     help="with --tp-shard: all-reduces by the peer-to-peer kernels in loop-back form")
+    ap.add_argument("--family", default="natilix", choices=["natilix", "pelenex"],
+                    help="with --hybrid: which hybrid family is measured (pelenex: next to natilix "
+                         "and dense)")
     ap.add_argument("--hybrid", default="",
                     help="instead of the headline workload: the hybrid family (Natilix) next to "
                          "the dense decoder of equal size; comma-separated sizes of "

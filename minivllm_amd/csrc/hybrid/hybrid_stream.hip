@@ -117,8 +117,10 @@ __global__ void unit_norm_store_kernel(T* __restrict__ q, const T* __restrict__ 
 }
 
 // gu row = [gate columns C | up columns C], C = NE * ff + sff.  act[t, c] = silu(w g) * (w u) with
-// w = dense[t, c / ff] for routed columns, 1 for the shared ones; exactly zero where w is.
-template <typename T>
+// w = dense[t, c / ff] for routed columns, 1 for the shared ones; exactly zero where w is (those
+// columns' inputs are not even read).  VEC consecutive columns per thread (one expert lookup per
+// run; VEC divides ff, sff and the row strides).
+template <typename T, int VEC>
 __global__ void swiglu_route_scale_kernel(const T* __restrict__ gu, long gu_stride,
                                           const float* __restrict__ dense, T* __restrict__ act,
                                           int NE, int ff, int C) {
@@ -126,11 +128,20 @@ __global__ void swiglu_route_scale_kernel(const T* __restrict__ gu, long gu_stri
     const T* g = gu + t * gu_stride;
     const T* u = g + C;
     const int routed = NE * ff;
-    for (int c = blockIdx.x * blockDim.x + threadIdx.x; c < C; c += gridDim.x * blockDim.x) {
+    for (int c = (blockIdx.x * blockDim.x + threadIdx.x) * VEC; c < C; c += gridDim.x * blockDim.x * VEC) {
         const float w = (dense && c < routed) ? dense[t * NE + c / ff] : 1.f;
-        float v = 0.f;
-        if (w != 0.f) v = siluf_(ld(g + c) * w) * (ld(u + c) * w);
-        st(act + t * (long)C + c, v);
+        float gv[VEC], uv[VEC];
+        if (w != 0.f) {
+            if constexpr (VEC == 1) { gv[0] = ld(g + c); uv[0] = ld(u + c); }
+            else { load_run<T, VEC>(g + c, gv); load_run<T, VEC>(u + c, uv); }
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) gv[j] = siluf_(gv[j] * w) * (uv[j] * w);
+        } else {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) gv[j] = 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) st(act + t * (long)C + c + j, gv[j]);
     }
 }
 
@@ -191,15 +202,23 @@ int hyb_swiglu_route_scale(const void* gu, long gu_stride, const void* dense, vo
                            int NE, int ff, int sff, int dt, hipStream_t s) {
     const int C = NE * ff + sff;
     if (T_ <= 0 || C <= 0) return 0;
-    if (T_ > 65535L * 32768L) return 1;
-    const int bx = (C + 255) / 256 > 64 ? 64 : (C + 255) / 256;
-    // blockIdx.y is limited to 65535 rows per launch
-    for (long t0 = 0; t0 < T_; t0 += 65535) {
+    const int esize = dt == 0 ? 2 : 4;
+    // eight columns per thread when every run of eight is one expert's and 16-byte addressable
+    const bool vec = (NE == 0 || ff % 8 == 0) && sff % 8 == 0 && gu_stride % 8 == 0 &&
+                     (size_t)gu % (4 * esize) == 0 && (C * (size_t)esize) % (4 * esize) == 0;
+    const int per = vec ? 8 : 1;
+    const int need = (C / per + 255) / 256;
+    const int bx = need > 64 ? 64 : (need < 1 ? 1 : need);
+    for (long t0 = 0; t0 < T_; t0 += 65535) {          // blockIdx.y holds at most 65535 rows
         const long n = T_ - t0 < 65535 ? T_ - t0 : 65535;
-        HYB_DISPATCH(dt, hipLaunchKernelGGL(swiglu_route_scale_kernel<T>, dim3(bx, n), dim3(256), 0, s,
-                                            (const T*)gu + t0 * gu_stride,
-                                            gu_stride, dense ? (const float*)dense + t0 * NE : nullptr,
-                                            (T*)act + t0 * (long)C, NE, ff, C));
+#define SWI(VEC)                                                                                  \
+        HYB_DISPATCH(dt, hipLaunchKernelGGL((swiglu_route_scale_kernel<T, VEC>), dim3(bx, n),      \
+                                            dim3(256), 0, s, (const T*)gu + t0 * gu_stride,       \
+                                            gu_stride,                                            \
+                                            dense ? (const float*)dense + t0 * NE : nullptr,      \
+                                            (T*)act + t0 * (long)C, NE, ff, C))
+        if (vec) SWI(8); else SWI(1);
+#undef SWI
     }
     return HYB_LAUNCH_OK();
 }

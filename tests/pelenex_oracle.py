@@ -164,17 +164,18 @@ def gated_ff(x, p):
 
 def feed_forward(h, p, f, margins=None):
     """``margins`` (a list of length T): lowered to the gap between the last chosen and the best
-    rejected score of every token (how close the routing decision is)."""
+    rejected router logit of every token (how close the routing decision is)."""
     if f["kind"] == "dense":
         return gated_ff(h, p)
     n, top = f["router"]["experts"], f["router"]["top"]
-    s = torch.sigmoid(lin(p["router"], h))
+    z = lin(p["router"], h)
+    s = torch.sigmoid(z)
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         ranked = sorted(range(n), key=lambda e: (-float(s[t, e]), e))
         order = ranked[:top]
         if margins is not None and top < n:
-            margins[t] = min(margins[t], float(s[t, ranked[top - 1]] - s[t, ranked[top]]))
+            margins[t] = min(margins[t], float(z[t, ranked[top - 1]] - z[t, ranked[top]]))
         for e in order:
             pe = {k[len(f"e{e}."):]: v for k, v in p.items() if k.startswith(f"e{e}.")}
             out[t] += gated_ff(s[t, e] * h[t], pe)
