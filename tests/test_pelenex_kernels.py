@@ -198,8 +198,11 @@ def _two_steps(run, S, lens1, lens2, slots):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("lanes", ["4", "8", "16", ""])
 @pytest.mark.parametrize("H,D,E", [(3, 48, 48), (2, 16, 80), (1, 130, 24), (4, 64, 64)])
-def test_mlstm_and_gla_scans(dt, H, D, E):
+def test_mlstm_and_gla_scans(dt, H, D, E, lanes, monkeypatch):
+    """``lanes``: lanes per state column of the scan kernel (empty: its own choice)."""
+    monkeypatch.setenv("MINIVLLM_SCAN_LPC", lanes)
     torch.manual_seed(4)
     S = 5
     lens1, lens2, slots = [37, 1, 0, 20], [3, 18, 0, 1], [4, 0, -1, 2]
@@ -235,8 +238,10 @@ def test_mlstm_and_gla_scans(dt, H, D, E):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("lanes", ["4", "8", "16"])
 @pytest.mark.parametrize("H,G,D,E,taps", [(4, 2, 32, 32, 3), (2, 2, 24, 40, 4), (3, 1, 130, 16, 1)])
-def test_channel_delta(dt, H, G, D, E, taps):
+def test_channel_delta(dt, H, G, D, E, taps, lanes, monkeypatch):
+    monkeypatch.setenv("MINIVLLM_SCAN_LPC", lanes)
     torch.manual_seed(5)
     S = 5
     lens1, lens2, slots = [37, 1, 0, 20], [3, 18, 0, 1], [4, 0, -1, 2]
