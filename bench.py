@@ -377,10 +377,12 @@ def pelenex_comparison(args) -> dict:
         natilix, dense = hybrid_models(size)
         row = {}
         for name, model in (("pelenex", pelenex_model(size)), ("natilix", natilix), ("dense", dense)):
+            if args.only and name != args.only:
+                continue                         # (a kernel trace of one model)
             r = bench_model(args, model, 0, 1)
             row[name] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in r.items() if k in keep}
         for k in ("prefill_tok_s", "decode_tok_s"):
-            if all(k in row[n] for n in ("pelenex", "natilix", "dense")):
+            if all(n in row and k in row[n] for n in ("pelenex", "natilix", "dense")):
                 row[f"pelenex_over_natilix_{k}"] = round(row["pelenex"][k] / row["natilix"][k], 3)
                 row[f"pelenex_over_dense_{k}"] = round(row["pelenex"][k] / row["dense"][k], 3)
         out["sizes"][size] = row
@@ -689,6 +691,8 @@ def main():
     ap.add_argument("--family", default="natilix", choices=["natilix", "pelenex"],
                     help="with --hybrid: which hybrid family is measured (pelenex: next to natilix "
                          "and dense)")
+    ap.add_argument("--only", default="", choices=["", "pelenex", "natilix", "dense"],
+                    help="with --hybrid --family pelenex: measure this one model only")
     ap.add_argument("--hybrid", default="",
                     help="instead of the headline workload: the hybrid family (Natilix) next to "
                          "the dense decoder of equal size; comma-separated sizes of "

@@ -131,9 +131,9 @@ __global__ void gated_head_norm_kernel(const float* __restrict__ o, const float*
 }
 
 // One workgroup (256 threads) per token: fp32 router logits (the row is read once, eight experts'
-// partial sums per pass), softmax over all experts (sig: sigmoid of each logit), best `keep` of `groups` groups (a group
-// scores its best expert), `top` largest eligible scores; dense [T, NE] out, zero where not
-// chosen.  Ties go to the lower index.  LDS: 2 * NE + 32 floats.
+// partial sums per pass), softmax over all experts (sig: the sigmoid of each logit instead), best
+// `keep` of `groups` groups (a group scores its best expert), `top` largest eligible scores; dense
+// [T, NE] out, zero where not chosen.  Ties go to the lower index.  LDS: 2 * NE + 32 floats.
 template <typename T>
 __global__ void grouped_route_kernel(const T* __restrict__ h, const float* __restrict__ wr,
                                      float* __restrict__ dense, int W, int NE, int top,

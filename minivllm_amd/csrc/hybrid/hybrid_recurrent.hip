@@ -97,30 +97,54 @@ __global__ void __launch_bounds__(256) gated_scan_kernel(const ScanArgs a) {
     const TI* vp = (const TI*)a.v;
 
     if (n == 1) {
-        // A single token (decode rows, one-token portions): no staging - every lane reads its own
-        // slice of k, q (and the decay) and its column's v straight from memory, updates, reduces.
+        // A single token (decode rows, one-token portions): k, q and the decay vector of the head
+        // (and MLSTM's three factors) are worked out once per workgroup into LDS, every lane then
+        // takes its slice and its column's v, updates, reduces.  No chunk machinery.
         const long t = first;
+        constexpr int DP = LPC * NR;
+        for (int i = tid; i < NIMG * DP; i += 256) {
+            const int which = i / DP, d = i - which * DP;
+            float v = 0.f;
+            if (d < D) {
+                if (which == 0) v = ld(kp + t * a.k_row + (long)g * D + d);
+                else if (which == 1) v = ld(qp + t * a.q_row + (long)g * D + d) * a.qscale;
+                else if constexpr (MODE == GLA)
+                    v = expf(logsigmoidf_(ld((const TI*)a.a + t * a.a_row + (long)h * D + d) +
+                                          a.a_bias[h * D + d]) * a.tau_inv);
+                else if constexpr (MODE == CDELTA) v = ((const float*)a.a)[t * a.a_row + (long)h * D + d];
+            }
+            sm[i] = v;
+        }
+        if constexpr (MODE == MLSTM) {
+            if (tid == 0) {
+                const float gi = a.cap * tanhf((ld((const TI*)a.gi + t * a.g_row + h) + a.bi[h]) / a.cap);
+                const float gf = logsigmoidf_(a.cap * tanhf((ld((const TI*)a.gf + t * a.g_row + h) + a.bf[h]) / a.cap));
+                const float m2 = fmaxf(gf + m_run, gi);
+                sm[NIMG * DP] = expf(gf + m_run - m2);
+                sm[NIMG * DP + 1] = expf(gi - m2);
+                sm[NIMG * DP + 2] = expf(-m2);
+                sm[NIMG * DP + 3] = m2;
+            }
+        }
+        __syncthreads();
         float kk[NR], qq[NR], gg[MODE == MLSTM ? 1 : NR];
 #pragma unroll
-        for (int i = 0; i < NR; ++i) {
-            const int d = d0 + i;
-            const bool in = d < D;
-            kk[i] = in ? ld(kp + t * a.k_row + (long)g * D + d) : 0.f;
-            qq[i] = in ? ld(qp + t * a.q_row + (long)g * D + d) * a.qscale : 0.f;
-            if constexpr (MODE == GLA)
-                gg[i] = in ? expf(logsigmoidf_(ld((const TI*)a.a + t * a.a_row + (long)h * D + d) +
-                                               a.a_bias[h * D + d]) * a.tau_inv) : 0.f;
-            if constexpr (MODE == CDELTA) gg[i] = in ? ((const float*)a.a)[t * a.a_row + (long)h * D + d] : 0.f;
+        for (int i = 0; i < NR / 4; ++i) {
+            const float4 k4 = reinterpret_cast<const float4*>(sm + d0)[i];
+            const float4 q4 = reinterpret_cast<const float4*>(sm + DP + d0)[i];
+            kk[4 * i] = k4.x; kk[4 * i + 1] = k4.y; kk[4 * i + 2] = k4.z; kk[4 * i + 3] = k4.w;
+            qq[4 * i] = q4.x; qq[4 * i + 1] = q4.y; qq[4 * i + 2] = q4.z; qq[4 * i + 3] = q4.w;
+            if constexpr (MODE != MLSTM) {
+                const float4 g4 = reinterpret_cast<const float4*>(sm + 2 * DP + d0)[i];
+                gg[4 * i] = g4.x; gg[4 * i + 1] = g4.y; gg[4 * i + 2] = g4.z; gg[4 * i + 3] = g4.w;
+            }
         }
         const float ve = col ? ld(vp + t * a.v_row + (long)h * E + e) : 0.f;
         float po = 0.f, pn = 0.f, em = 0.f;
         if constexpr (MODE == MLSTM) {
-            const float gi = a.cap * tanhf((ld((const TI*)a.gi + t * a.g_row + h) + a.bi[h]) / a.cap);
-            const float gf = logsigmoidf_(a.cap * tanhf((ld((const TI*)a.gf + t * a.g_row + h) + a.bf[h]) / a.cap));
-            const float m2 = fmaxf(gf + m_run, gi);
-            const float fs = expf(gf + m_run - m2), is = expf(gi - m2);
-            em = expf(-m2);
-            m_run = m2;
+            const float fs = sm[NIMG * DP], is = sm[NIMG * DP + 1];
+            em = sm[NIMG * DP + 2];
+            m_run = sm[NIMG * DP + 3];
             const float kv = is * ve;
 #pragma unroll
             for (int i = 0; i < NR; ++i) {
