@@ -228,17 +228,20 @@ def _standout_model(size, keep, bs):
 
 @pytest.mark.parametrize("device,dtype", CASES)
 @pytest.mark.parametrize("decoded", [False, True], ids=["prompt", "decoded"])
-def test_keys_at_every_edge(tmp_path, device, dtype, decoded):
+@pytest.mark.parametrize("n", [41, 300], ids=["short", "far"])
+def test_keys_at_every_edge(tmp_path, device, dtype, decoded, n):
     """Token 38 sits at a key position, token 39 at the query position (the last one); key
     positions: the very first token, the last kept one and the first not kept, both sides of a
     block border, far back but kept, just inside and just outside the window.  The oracle's logits
     for a key on either side of an edge differ widely, so a window or a kept prefix that is off by
     one cannot pass."""
-    size, keep, bs, n = 11, 4, 8, 41
+    size, keep, bs = 11, 4, 8
     c, w = _standout_model(size, keep, bs)
     q = n - 1
     places = [0, keep - 1, keep, bs - 1, bs, 2 * bs - 1, q - size + 1, q - size, q - 1]
-    eng = make_engine(tmp_path, c, w, device, dtype, blocks=12, block_size=bs, seqs=2)
+    if n > 100:                      # the kept tokens are hundreds of positions back
+        places = [0, keep - 1, keep, q - size + 1, q - size]
+    eng = make_engine(tmp_path, c, w, device, dtype, blocks=n // bs + 4, block_size=bs, seqs=2)
     seen_logits = {}
     for j in places:
         toks = [1 + (t * 7) % 37 for t in range(n)]            # ids 1 .. 37
