@@ -294,6 +294,48 @@ def test_sizes_that_happen_to_be_one_or_equal(tmp_path, device, dtype):
         eng.exit()
 
 
+def _random_config(seed):
+    """A configuration drawn from a seed: widths, head counts and sizes (also odd multiples and
+    sizes above 128), layer order, windows, taps, experts, groups and constants all vary."""
+    g = torch.Generator().manual_seed(seed)
+
+    def pick(*xs):
+        return xs[int(torch.randint(0, len(xs), (1,), generator=g))]
+    width = pick(24, 48, 96, 160)
+    layers = []
+    for _ in range(pick(2, 3, 4, 5)):
+        kind = pick("mlstm", "parallel", "delta")
+        if kind == "mlstm":
+            m = fx.mlstm(heads=pick(1, 2, 5), dim=pick(8, 20, 40, 136), vdim=pick(8, 28, 72), cap=pick(2.0, 9.0, 15.0))
+        elif kind == "parallel":
+            kv = pick(1, 2, 3)
+            m = fx.parallel(heads=kv * pick(1, 2, 4), kv_heads=kv, dim=pick(8, 24, 40, 72, 144),
+                            size=pick(1, 5, 16, 33, 500), keep=pick(0, 1, 7, 20), scale=pick(0.3, 1.1),
+                            rheads=pick(1, 3), rdim=pick(4, 12, 40), rvdim=pick(8, 36, 132), tau=pick(1.0, 4.0, 16.0))
+        else:
+            kv = pick(1, 2)
+            m = fx.delta(heads=kv * pick(1, 3), kv_heads=kv, dim=pick(8, 20, 48, 136), vdim=pick(8, 24, 68),
+                         conv=pick(1, 2, 3, 4, 5))
+        f = pick(None, fx.dense(pick(16, 40, 104)),
+                 fx.moe(ff=pick(8, 24, 40), experts=pick(2, 5, 16), top=pick(1, 2), shared=pick(0, 8, 56)))
+        layers.append((m, f))
+    return fx.config(layers, width=width, vocab=pick(50, 131), eps=pick(1e-6, 1e-5),
+                     groups=pick(1, 2, 4, 8), softcap=pick(0.0, 7.0, 30.0))
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+@pytest.mark.parametrize("seed", list(range(8)))
+def test_configurations_drawn_at_random(tmp_path, device, dtype, seed):
+    c = _random_config(seed)
+    w = fx.weights(c, 70 + seed, rank=3 + seed % 4)
+    toks = tokens(45, c["vocab"], 80 + seed)
+    eng = make_engine(tmp_path, c, w, device, dtype, blocks=16, block_size=8)
+    want = Expected(c, w, toks)
+    close(run_schedule(eng, {"a": toks}, [[("a", 45)]])["a"], want, dtype)
+    close(run_schedule(eng, {"b": toks}, [[("b", 7)], [("b", 2)], [("b", 26)]] + [[("b", 1)]] * 10)["b"], want, dtype)
+    eng.exit()
+
+
 def _follow(c, w, prompt, gen, dtype):
     """Greedy tokens against the oracle (recomputed from scratch per token: it keeps no state)."""
     toks = list(prompt)
