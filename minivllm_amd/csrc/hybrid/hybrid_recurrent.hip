@@ -44,7 +44,7 @@ struct ScanArgs {
     const float *bi, *bf;           // MLSTM [H]
     float cap;
     const float* beta;              // CDELTA [T, H]
-    float *state, *nstate, *mstate; // [slots,H,D,E], MLSTM: [slots,H,D], [slots,H]
+    float *state, *nstate, *mstate; // [slots,H,D,E]; MLSTM: [slots,H,ZG,D], [slots,H,ZG], ZG = ceil(E/16)
     const int *cu_q, *positions, *slots;
     float* o;                       // [T, H, E]
     int H, G, D, E;
@@ -80,6 +80,12 @@ __global__ void __launch_bounds__(256) gated_scan_kernel(const ScanArgs a) {
     const int g = h / (H / G);
     const int d0 = r * NR;
     const bool has_past = a.positions[first] > 0;
+    // MLSTM's normaliser n and running maximum m are the same for every column, but the workgroups
+    // of one (sequence, head) - one per block of columns - each read them when they start and would
+    // overwrite them when they end: so the slot keeps one copy per 16 columns (the smallest block),
+    // and a workgroup reads the copy of its first 16 columns and writes those of all it covers
+    const int ZG = (E + 15) / 16, zg0 = e0 / 16;
+    constexpr int NZG = COLS / 16;
     float S[NR], N[MODE == MLSTM ? NR : 1];
     float* sp = a.state + (((long)slot * H + h) * D) * E + (col ? e : 0);
 #pragma unroll
@@ -87,10 +93,10 @@ __global__ void __launch_bounds__(256) gated_scan_kernel(const ScanArgs a) {
         S[i] = (has_past && col && d0 + i < D) ? sp[(long)(d0 + i) * E] : 0.f;
     float m_run = 0.f;
     if constexpr (MODE == MLSTM) {
-        const float* np = a.nstate + ((long)slot * H + h) * D;
+        const float* np = a.nstate + (((long)slot * H + h) * ZG + zg0) * D;
 #pragma unroll
         for (int i = 0; i < NR; ++i) N[i] = (has_past && d0 + i < D) ? np[d0 + i] : 0.f;
-        if (has_past) m_run = a.mstate[(long)slot * H + h];
+        if (has_past) m_run = a.mstate[((long)slot * H + h) * ZG + zg0];
     }
     const TI* qp = (const TI*)a.q;
     const TI* kp = (const TI*)a.k;
@@ -190,12 +196,12 @@ __global__ void __launch_bounds__(256) gated_scan_kernel(const ScanArgs a) {
                 if (d0 + i < D) sp[(long)(d0 + i) * E] = S[i];
         }
         if constexpr (MODE == MLSTM) {
-            if (blockIdx.z == 0 && c == 0) {
-                float* np = a.nstate + ((long)slot * H + h) * D;
+            if (c < NZG && zg0 + c < ZG) {              // (these lanes sit in wave 0, which owns m_run)
+                float* np = a.nstate + (((long)slot * H + h) * ZG + zg0 + c) * D;
 #pragma unroll
                 for (int i = 0; i < NR; ++i)
                     if (d0 + i < D) np[d0 + i] = N[i];
-                if (tid == 0) a.mstate[(long)slot * H + h] = m_run;
+                if (r == 0) a.mstate[((long)slot * H + h) * ZG + zg0 + c] = m_run;
             }
         }
         return;
@@ -431,12 +437,12 @@ __global__ void __launch_bounds__(256) gated_scan_kernel(const ScanArgs a) {
             if (d0 + i < D) sp[(long)(d0 + i) * E] = S[i];
     }
     if constexpr (MODE == MLSTM) {
-        if (blockIdx.z == 0 && c == 0) {
-            float* np = a.nstate + ((long)slot * H + h) * D;
+        if (c < NZG && zg0 + c < ZG) {              // (these lanes sit in wave 0, which owns m_run)
+            float* np = a.nstate + (((long)slot * H + h) * ZG + zg0 + c) * D;
 #pragma unroll
             for (int i = 0; i < NR; ++i)
                 if (d0 + i < D) np[d0 + i] = N[i];
-            if (tid == 0) a.mstate[(long)slot * H + h] = m_run;
+            if (r == 0) a.mstate[((long)slot * H + h) * ZG + zg0 + c] = m_run;
         }
     }
 }
@@ -507,8 +513,8 @@ int hyb_gla_scan(const void* q, const void* k, const void* v, long q_row, long k
     return 1;
 }
 
-// gi, gf [T, H] raw gate projections (activation type, element stride g_row); nstate [slots, H, D],
-// mstate [slots, H].
+// gi, gf [T, H] raw gate projections (activation type, element stride g_row); nstate
+// [slots, H, ZG, D], mstate [slots, H, ZG] with ZG = ceil(E / 16) identical copies.
 int hyb_mlstm_scan(const void* q, const void* k, const void* v, long q_row, long k_row, long v_row,
                    const void* gi, const void* gf, long g_row, const void* bi, const void* bf,
                    float cap, void* state, void* nstate, void* mstate, const void* cu_q,

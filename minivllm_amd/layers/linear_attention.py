@@ -47,12 +47,15 @@ class MatrixLSTM(nn.Module):
         self.f_bias = nn.Parameter(torch.zeros(H, **f32), requires_grad=False)
         self.norm_weight = nn.Parameter(torch.ones(H * E, **f32), requires_grad=False)
         self.state: Optional[torch.Tensor] = None          # [slots, H, D, E]
-        self.norm_state: Optional[torch.Tensor] = None     # [slots, H, D]
-        self.max_state: Optional[torch.Tensor] = None      # [slots, H]
+        self.norm_state: Optional[torch.Tensor] = None     # [slots, H, Z, D], Z = ceil(E / 16) copies
+        self.max_state: Optional[torch.Tensor] = None      # [slots, H, Z]
 
     def state_spec(self):
+        """n and m are kept once per 16 value columns: the scan kernel's workgroups (one per block
+        of columns of a head) each read and write their own copy, so none sees another's update."""
         H, D, E = self.num_heads, self.head_dim, self.v_head_dim
-        return [("state", (H, D, E)), ("norm_state", (H, D)), ("max_state", (H,))]
+        Z = (E + 15) // 16
+        return [("state", (H, D, E)), ("norm_state", (H, Z, D)), ("max_state", (H, Z))]
 
     def split_sizes(self):
         """Column blocks of the fused input projection: q, k, v, output gate, input gate, forget gate."""

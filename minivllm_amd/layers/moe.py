@@ -45,7 +45,7 @@ class RoutedGatedExperts(nn.Module):
     feed-forward of size ``shared_ff``.
 
     Router: s = sigmoid(W_r h) in fp32, the ``top`` largest scores chosen (ties to the lower
-    index) and used as weights as they are.  The weight multiplies the expert's INPUT:
+    index) and used as weights as they are.  An expert is fed its weight times the row:
     out = sum_j expert_j(s_j h) + shared(h).
 
     Execution: one stacked gate+up weight [2 C, W], C = experts * ff + shared_ff (all gate rows,

@@ -448,7 +448,9 @@ def mlstm_scan(q, k, v, i_raw, f_raw, i_bias, f_bias, cap, state, norm_state, ma
                cu_q, positions, slots):
     T, H, D = q.shape
     E = v.shape[2]
-    assert state.shape[1:] == (H, D, E) and norm_state.shape[1:] == (H, D) and max_state.shape[1:] == (H,)
+    ZG = (E + 15) // 16
+    assert state.shape[1:] == (H, D, E) and norm_state.shape[1:] == (H, ZG, D) \
+        and max_state.shape[1:] == (H, ZG)
     assert i_raw.shape == (T, H) and f_raw.shape == (T, H) and i_raw.stride(1) == 1 and f_raw.stride(1) == 1
     assert T == 1 or i_raw.stride(0) == f_raw.stride(0)
     assert k.dtype == q.dtype and v.dtype == q.dtype and i_raw.dtype == q.dtype and f_raw.dtype == q.dtype

@@ -361,8 +361,9 @@ def mlstm_scan(q, k, v, i_raw, f_raw, i_bias, f_bias, cap, state, norm_state, ma
     i = cap tanh((i_raw + b_i) / cap), f = logsigmoid(cap tanh((f_raw + b_f) / cap)),
     m' = max(f + m, i); S <- e^(f+m-m') S + e^(i-m') k v^T; n likewise with k alone;
     o = S^T q / (max(|n . q|, e^(-m')) + 1e-6), q scaled by D^-1/2.  q, k [T,H,D]; v [T,H,E];
-    gates [T,H]; ``state`` [slots,H,D,E], ``norm_state`` [slots,H,D], ``max_state`` [slots,H]
-    fp32.  Returns o [T,H,E] fp32."""
+    gates [T,H]; ``state`` [slots,H,D,E] fp32; ``norm_state`` [slots,H,Z,D] and ``max_state``
+    [slots,H,Z] fp32 hold Z = ceil(E/16) identical copies of n and m (the GPU kernel's workgroups,
+    one per block of columns, each read and write their own).  Returns o [T,H,E] fp32."""
     T, H, D = q.shape
     E = v.shape[2]
     qf, kf, vf = q.float() * D ** -0.5, k.float(), v.float()
@@ -371,8 +372,8 @@ def mlstm_scan(q, k, v, i_raw, f_raw, i_bias, f_bias, cap, state, norm_state, ma
     o = torch.zeros(T, H, E, dtype=torch.float32)
     for s, e, slot, past in _seq_rows(cu_q, positions, slots):
         S = state[slot].clone() if past else torch.zeros(H, D, E)
-        n = norm_state[slot].clone() if past else torch.zeros(H, D)
-        m = max_state[slot].clone() if past else torch.zeros(H)
+        n = norm_state[slot][:, 0].clone() if past else torch.zeros(H, D)
+        m = max_state[slot][:, 0].clone() if past else torch.zeros(H)
         for t in range(s, e):
             m2 = torch.maximum(fg[t] + m, ig[t])
             a, b = torch.exp(fg[t] + m - m2), torch.exp(ig[t] - m2)
@@ -381,7 +382,9 @@ def mlstm_scan(q, k, v, i_raw, f_raw, i_bias, f_bias, cap, state, norm_state, ma
             m = m2
             den = torch.maximum((n * qf[t]).sum(-1).abs(), torch.exp(-m)) + 1e-6
             o[t] = torch.einsum("hde,hd->he", S, qf[t]) / den[:, None]
-        state[slot], norm_state[slot], max_state[slot] = S, n, m
+        state[slot] = S
+        norm_state[slot] = n[:, None, :]
+        max_state[slot] = m[:, None]
     return o
 
 

@@ -199,7 +199,7 @@ def _two_steps(run, S, lens1, lens2, slots):
 
 @pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("lanes", ["4", "8", "16", ""])
-@pytest.mark.parametrize("H,D,E", [(3, 48, 48), (2, 16, 80), (1, 130, 24), (4, 64, 64)])
+@pytest.mark.parametrize("H,D,E", [(3, 48, 48), (2, 16, 80), (1, 130, 24), (4, 64, 64), (2, 32, 168)])
 def test_mlstm_and_gla_scans(dt, H, D, E, lanes, monkeypatch):
     """``lanes``: lanes per state column of the scan kernel (empty: its own choice)."""
     monkeypatch.setenv("MINIVLLM_SCAN_LPC", lanes)
@@ -211,7 +211,9 @@ def test_mlstm_and_gla_scans(dt, H, D, E, lanes, monkeypatch):
     for p in projs:
         p[:, 2 * H * D + H * E:2 * H * D + H * E + 2 * H] *= 6       # gates that reach the cap
     bi, bf, ab = torch.randn(H), 2 + torch.randn(H), torch.randn(H * D)
-    init = [torch.randn(S, H, D, E), torch.randn(S, H, D), torch.randn(S, H), torch.randn(S, H, D, E)]
+    Z = (E + 15) // 16             # copies of the normaliser and the running maximum per head
+    init = [torch.randn(S, H, D, E), torch.randn(S, H, 1, D).expand(S, H, Z, D).contiguous(),
+            torch.randn(S, H, 1).expand(S, H, Z).contiguous(), torch.randn(S, H, D, E)]
     res = {}
     for name, mod, to in (("cpu", ref, lambda t: t), ("gpu", hk, lambda t: t.cuda())):
         st = [to(t.clone()) for t in init]
