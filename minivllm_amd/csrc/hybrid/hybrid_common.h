@@ -1,5 +1,5 @@
-// Helpers shared by the kernels of hybrid decoders (fp32 residual stream, zero-centred norms,
-// attention with a sink, gated delta rule, grouped expert routing).  Activations are bfloat16
+// Helpers shared by the kernels of hybrid decoders (fp32 residual stream, zero-centred or grouped
+// norms, attention with a sink or a window, gated outer-product recurrences, expert routing).  Activations are bfloat16
 // or float (template parameter), everything a norm, a softmax or a recurrence touches is fp32.
 #pragma once
 #include <hip/hip_runtime.h>

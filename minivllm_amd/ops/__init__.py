@@ -229,8 +229,9 @@ def sample(logits, temperatures, seed=0, step=0, generator=None):
 
 
 # ------------------------------------------------------------------ hybrid decoders
-# (fp32 residual stream with zero-centred norms, pair rotation + value mixing, attention with a
-# sink, gated delta rule, grouped expert routing).  GPU tensors go to the kernels of
+# (fp32 residual stream with zero-centred or grouped norms, pair rotation + value mixing or
+# sinusoidal positions, attention with a sink / a window / a distance penalty, gated delta rule,
+# gated linear attention, matrix LSTM, grouped or sigmoid expert routing).  GPU tensors go to the kernels of
 # ``csrc/hybrid`` (their own library, ``ops.hip_hybrid``), CPU tensors to ``torch_seqmix``.
 from . import torch_seqmix
 

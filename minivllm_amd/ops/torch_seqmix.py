@@ -1,7 +1,10 @@
 """Plain PyTorch forms of the ops that hybrid decoders add to the dense ones: norms with a
 zero-centred weight around a fp32 residual stream, rotation of neighbouring pairs with value
-mixing, attention with a sink term and separate key / value head sizes, the gated delta rule
-with its short convolutions, and routing over grouped experts.  They run CPU tensors (the
+mixing, attention with a sink term and separate key / value head sizes (optionally windowed,
+with kept first tokens and a distance penalty), the gated delta rule with its short
+convolutions, routing over grouped experts; and, for decoders with parallel sublayers, grouped
+norms, sinusoidal positions, gated linear attention, the matrix LSTM and sigmoid-routed gated
+experts.  They run CPU tensors (the
 engine's CPU mode) and serve as the shape-for-shape counterpart of the gfx950 kernels in
 ``csrc/hybrid`` (``ops.hip_hybrid``).  Everything a recurrence touches is fp32 here too.
 
