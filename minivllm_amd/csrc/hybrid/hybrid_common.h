@@ -1,6 +1,7 @@
 // Helpers shared by the kernels of hybrid decoders (fp32 residual stream, zero-centred or grouped
-// norms, attention with a sink or a window, gated outer-product recurrences, expert routing).  Activations are bfloat16
-// or float (template parameter), everything a norm, a softmax or a recurrence touches is fp32.
+// norms, attention with a sink or a window, gated outer-product recurrences, expert routing).
+// Activations are bfloat16 or float (template parameter), everything a norm, a softmax or a
+// recurrence touches is fp32.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
